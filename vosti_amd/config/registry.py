@@ -115,12 +115,15 @@ class NativeConfig:
 
 
 def resolve_architecture(raw: Mapping[str, Any]) -> str:
-    """The architecture that a config.json names: the first entry of "architectures", else a registered
-    "model_type"."""
+    """The architecture that a config.json names: a registered "architecture", else the first entry of
+    "architectures", else a registered "model_type"."""
     archs = raw.get("architectures")
+    types = model_types()
+    # A configuration may also name its architecture with a plain string.
+    if isinstance(raw.get("architecture"), str) and (raw["architecture"] in _ARCHITECTURES or raw["architecture"] in types.values()):
+        return raw["architecture"]
     if isinstance(archs, (list, tuple)) and archs:
         return archs[0]
-    types = model_types()
     if raw.get("model_type") in types:
         return types[raw["model_type"]]
     raise ConfigError("config.json names no architecture (key 'architectures') and no known 'model_type'")

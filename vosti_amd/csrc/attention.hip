@@ -67,6 +67,11 @@ struct AttnArgs {
   float* part_acc;        // decode: [n_items * nq * nseg, d]
   int bt_stride, nq, nkv, d, P, window, nseg;
   float scale_log2;
+  // The variant with capped scores, kept first keys and a sink (see "Capped scores" below); unset for the others.
+  int keep = 0;           // with a window: keys below `keep` stay visible however far back they lie
+  float scale = 0.f, softcap = 0.f;   // score = softcap * tanh(q.k * scale / softcap); softcap 0: score = q.k * scale
+  const void* sinks = nullptr;        // [nq] or null: exp(sinks[head]) joins the softmax's denominator, with no value
+  int sinks_f32 = 0;
 };
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
@@ -79,7 +84,8 @@ struct RowCtx {
   int64_t page_stride;
   int k_len, d, P, lp, r16, g;   // lp = log2(P)
   int lo, pos;             // this lane's row sees keys lo..pos
-  int wave_lo;             // smallest key any row of the wave sees
+  int wave_lo;             // smallest key of the window that any row of the wave sees
+  int keep = 0;            // keys below this are the sequence's own and visible although they lie before the window
   bool row_ok;
   float scale_log2;
 };
@@ -165,13 +171,13 @@ __device__ __forceinline__ void scale_state(f32x4 (&ACC)[NDT], float ca, bool fr
 // Keys outside [first, k_len) may lie in pages this sequence does not own
 // (never written, or given back once the window passed them): their values
 // are replaced by zero so that stale NaN or Inf cannot reach the sum.
-__device__ __forceinline__ void zero_unowned(frag_t (&vf)[KEY_SLABS], int kb, int g, int first, int k_len) {
+__device__ __forceinline__ void zero_unowned(frag_t (&vf)[KEY_SLABS], int kb, int g, int first, int k_len, int keep = 0) {
 #pragma unroll
   for (int ks = 0; ks < KEY_SLABS; ++ks) {
     const int k0 = kb + ks * VK_SLAB + g * VK_VEC;
 #pragma unroll
     for (int j = 0; j < VK_VEC; ++j)
-      if (k0 + j >= k_len || k0 + j < first) vf[ks][j] = (elem_t)0.f;
+      if (k0 + j >= k_len || (k0 + j < first && k0 + j >= keep)) vf[ks][j] = (elem_t)0.f;
   }
 }
 
@@ -875,6 +881,239 @@ __global__ __launch_bounds__(128, 2) void attn_decode_pair_kernel(AttnArgs a) {
   }
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// Capped scores, kept first keys, a sink, and probabilities that are not rounded.
+//
+// The same attention with four things more, each a parameter of the launch:
+//   softcap   score = softcap * tanh((q.k) * scale / softcap) before the softmax (0: score = (q.k) * scale);
+//   keep      with a window, the row at position p sees key j <= p if p - j < window or j < keep: the first keys of
+//             a sequence stay visible at their own positions, and their tiles are visited before the window's;
+//   sinks     exp(sinks[head]) is added to the softmax's denominator of every row of that head; it has no key and
+//             no value, and is neither scaled nor capped;
+//   weights   the probabilities meet the values as 32-bit numbers.  In the bfloat16 build a probability is split
+//             into three bfloat16 numbers whose sum is the 32-bit value exactly (8 significant bits each), and the
+//             matrix unit adds the three products in 32-bit: three MFMAs a slab instead of one.
+// The reduction order is the one of the kernels above: tiles of 64 keys at absolute positions, four to a segment,
+// segments folded in ascending order; the tiles between the kept keys and the window are left out, which changes
+// no sum.  So the result does not depend on how a sequence was cut into steps.
+#ifdef VK_BF16
+#define P_PARTS 3
+#else
+#define P_PARTS 1
+#endif
+#define LOG2E 1.4426950408889634f
+
+__device__ __forceinline__ float sink_term(const AttnArgs& a, int head, float M) {
+  return fast_exp2(__builtin_fmaf(load_weight(a.sinks, a.sinks_f32, head), LOG2E, -M));
+}
+
+// tile_probs for scores in natural units (already scaled and capped), with kept first keys and unrounded weights.
+__device__ __forceinline__ void tile_probs_ext(float (&sc)[S_PER_LANE], int kb, int g, bool row_ok, int lo, int pos, int keep,
+                                               float& M, float& L, float& ca, frag_t (&pf)[P_PARTS][KEY_SLABS]) {
+  float pr[S_PER_LANE];
+  float psum = 0.f;
+  bool vis[S_PER_LANE];
+  float tmax = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < S_PER_LANE; ++i) {
+    const int key = kb + (i / VK_VEC) * VK_SLAB + g * VK_VEC + (i % VK_VEC);
+    vis[i] = row_ok && key <= pos && (key >= lo || key < keep);
+    tmax = fmaxf(tmax, vis[i] ? sc[i] : -INFINITY);
+  }
+  tmax = fmaxf(tmax, lane_xor16(tmax));
+  tmax = fmaxf(tmax, lane_xor32(tmax));
+  const float m = tmax * LOG2E;             // -inf: the row sees no key of the tile
+  const float Mn = (!(M > -INFINITY) || m > M + MAX_STEP) ? m : M;
+  ca = Mn > -INFINITY ? fast_exp2(M - Mn) : 1.f;
+#pragma unroll
+  for (int i = 0; i < S_PER_LANE; ++i) {
+    pr[i] = vis[i] ? fast_exp2(__builtin_fmaf(sc[i], LOG2E, -Mn)) : 0.f;
+    psum = psum + pr[i];
+  }
+  psum = psum + lane_xor16(psum);
+  psum = psum + lane_xor32(psum);
+  L = __builtin_fmaf(L, ca, psum);
+  M = Mn;
+#pragma unroll
+  for (int ks = 0; ks < KEY_SLABS; ++ks) {
+#ifdef VK_BF16
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      // Each difference is exact: what rounding to 8 bits leaves of a 24-bit number has 16 bits, then 8.
+      const float p = pr[ks * 8 + j];
+      const __bf16 hi = (__bf16)p;
+      const float r1 = p - (float)hi;
+      const __bf16 mid = (__bf16)r1;
+      pf[0][ks][j] = hi;
+      pf[1][ks][j] = mid;
+      pf[2][ks][j] = (__bf16)(r1 - (float)mid);
+    }
+#else
+    pf[0][ks] = f32x4{pr[ks * 4 + 0], pr[ks * 4 + 1], pr[ks * 4 + 2], pr[ks * 4 + 3]};
+#endif
+  }
+}
+
+template <int NDT, int NQS, bool V_LATE>
+__device__ __forceinline__ void tile_step_ext(const RowCtx& c, float scale, float softcap, const frag_t (&qf)[NQS], int kb, float& M,
+                                              float& L, f32x4 (&ACC)[NDT]) {
+  frag_t kf[KSUB][NQS];
+  frag_t vf[NDT][KEY_SLABS];
+  load_keys<NQS, false>(c, kb, kf);
+  if (!V_LATE) load_values<NDT, false>(c, kb, vf);
+  float sc[S_PER_LANE];
+  tile_scores<NQS, false>(c, kf, qf, sc);
+  if (V_LATE) {
+    __builtin_amdgcn_sched_barrier(0);
+    load_values<NDT, false>(c, kb, vf);
+  }
+  if (softcap > 0.f) {
+    const float inner = scale / softcap;
+#pragma unroll
+    for (int i = 0; i < S_PER_LANE; ++i) sc[i] = softcap * tanhf(sc[i] * inner);
+  } else {
+#pragma unroll
+    for (int i = 0; i < S_PER_LANE; ++i) sc[i] = sc[i] * scale;
+  }
+  frag_t pf[P_PARTS][KEY_SLABS];
+  float ca;
+  const bool fresh = !(M > -INFINITY);
+  tile_probs_ext(sc, kb, c.g, c.row_ok, c.lo, c.pos, c.keep, M, L, ca, pf);
+  scale_state<NDT>(ACC, ca, fresh);
+  if (kb + TILE_KEYS > c.k_len || kb < c.wave_lo) {
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt)
+      if (dt * 16 < c.d) zero_unowned(vf[dt], kb, c.g, c.wave_lo, c.k_len, c.keep);
+  }
+#pragma unroll
+  for (int dt = 0; dt < NDT; ++dt) {
+    if (dt * 16 < c.d) {
+#pragma unroll
+      for (int ks = 0; ks < KEY_SLABS; ++ks) {
+#pragma unroll
+        for (int part = 0; part < P_PARTS; ++part) ACC[dt] = mma_slab(vf[dt][ks], pf[part][ks], ACC[dt]);
+      }
+    }
+  }
+}
+
+// Prompt rows: attn_prefill_kernel with the four things above.
+template <int DPAD>
+__global__ __launch_bounds__(256) void attn_prefill_ext_kernel(AttnArgs a, int heads_per_wg) {
+  constexpr int NDT = DPAD / 16, NQS = DPAD / VK_SLAB;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int G = a.nq / a.nkv;
+  const int groups_per_kv = (G + heads_per_wg - 1) / heads_per_wg;
+  const int kvh = blockIdx.y / groups_per_kv;
+  const int hg = (blockIdx.y - kvh * groups_per_kv) * heads_per_wg + wave;
+  if (hg >= G) return;
+  const int head = kvh * G + hg;
+  const int item = blockIdx.x / (ITEM_ROWS / 16);
+  const int seq = a.items[2 * item];
+  const int q_off = a.items[2 * item + 1] + (blockIdx.x % (ITEM_ROWS / 16)) * 16;
+  const int q_begin = a.cu_q[seq], q_len = a.cu_q[seq + 1] - q_begin;
+  if (q_off >= q_len) return;
+  const int k_len = a.k_len[seq];
+  RowCtx c;
+  init_ctx(c, a, seq, kvh, k_len);
+  c.r16 = lane & 15;
+  c.g = lane >> 4;
+  const int nvalid = min(16, q_len - q_off);
+  c.row_ok = c.r16 < nvalid;
+  const int tok = q_begin + q_off + c.r16;
+  const int pos0 = k_len - q_len + q_off;
+  c.pos = pos0 + c.r16;
+  c.lo = a.window > 0 ? max(0, c.pos - a.window + 1) : 0;
+  c.wave_lo = a.window > 0 ? max(0, pos0 - a.window + 1) : 0;
+  c.keep = a.window > 0 ? a.keep : 0;
+  const int keep_tiles = (c.keep + TILE_KEYS - 1) / TILE_KEYS;
+  const int tile_lo = c.wave_lo / TILE_KEYS, tile_hi = (pos0 + nvalid - 1) / TILE_KEYS;
+
+  frag_t qf[NQS];
+  load_q<NQS>(a, tok, head, c.row_ok, c.g, qf);
+
+  float M = -INFINITY, L = 0.f;
+  f32x4 ACC[NDT];
+#pragma unroll
+  for (int dt = 0; dt < NDT; ++dt) ACC[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int seg = keep_tiles > 0 ? 0 : tile_lo / SEG_TILES; seg <= tile_hi / SEG_TILES; ++seg) {
+    const int t_begin = seg * SEG_TILES, t_end = min(tile_hi, seg * SEG_TILES + SEG_TILES - 1);
+    if (t_begin >= keep_tiles && t_end < tile_lo) continue;      // between the kept keys and the window
+    float Ms = -INFINITY, Ls = 0.f;
+    f32x4 As[NDT];
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt) As[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int t = t_begin; t <= t_end; ++t)
+      if (t < keep_tiles || t >= tile_lo) tile_step_ext<NDT, NQS, true>(c, a.scale, a.softcap, qf, t * TILE_KEYS, Ms, Ls, As);
+    fold<NDT>(M, L, ACC, Ms, Ls, As);
+  }
+  if (c.row_ok) {
+    if (a.sinks != nullptr && M > -INFINITY) L = L + sink_term(a, head, M);
+    const float inv = L > 0.f ? 1.0f / L : 0.f;
+    elem_t* orow = a.out + ((int64_t)tok * a.nq + head) * a.d;
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt) {
+      if (dt * 16 < a.d) {
+        const float o[4] = {ACC[dt].x * inv, ACC[dt].y * inv, ACC[dt].z * inv, ACC[dt].w * inv};
+        elem_t* p = orow + dt * 16 + 4 * c.g;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) p[i] = from_f32<elem_t>(o[i]);
+      }
+    }
+  }
+}
+
+// Decoded tokens: attn_decode_plain_kernel with the four things above; attn_combine_kernel folds its segments.
+template <int DPAD, bool V_LATE>
+__global__ __launch_bounds__(64 * PLAIN_WAVES) void attn_decode_ext_kernel(AttnArgs a) {
+  constexpr int NDT = DPAD / 16, NQS = DPAD / VK_SLAB;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int G = a.nq / a.nkv, HT = (G + 15) >> 4;
+  const int kvh = blockIdx.y / HT, ht = blockIdx.y - kvh * HT;
+  const int seg = blockIdx.z * PLAIN_WAVES + wave;
+  const int seq = a.items[2 * blockIdx.x], q_off = a.items[2 * blockIdx.x + 1];
+  const int q_begin = a.cu_q[seq], q_len = a.cu_q[seq + 1] - q_begin;
+  const int k_len = a.k_len[seq];
+  const int tok = q_begin + q_off;
+  const int pos = k_len - q_len + q_off;
+  const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
+  const int keep = a.window > 0 ? a.keep : 0;
+  const int keep_tiles = (keep + TILE_KEYS - 1) / TILE_KEYS, tile_lo = lo / TILE_KEYS;
+  const int t0 = seg * SEG_TILES, t1 = min(pos / TILE_KEYS, seg * SEG_TILES + SEG_TILES - 1);
+  if (t0 > t1 || (t0 >= keep_tiles && t1 < tile_lo)) return;   // whole wave; no barrier follows
+
+  RowCtx c;
+  init_ctx(c, a, seq, kvh, k_len);
+  c.r16 = lane & 15;
+  c.g = lane >> 4;
+  c.row_ok = c.r16 < min(16, G - ht * 16);
+  c.pos = pos;
+  c.lo = lo;
+  c.wave_lo = lo;
+  c.keep = keep;
+  const int head = kvh * G + ht * 16 + c.r16;
+  frag_t qf[NQS];
+  load_q<NQS>(a, tok, head, c.row_ok, c.g, qf);
+  float M = -INFINITY, L = 0.f;
+  f32x4 ACC[NDT];
+#pragma unroll
+  for (int dt = 0; dt < NDT; ++dt) ACC[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  for (int t = t0; t <= t1; ++t)
+    if (t < keep_tiles || t >= tile_lo) tile_step_ext<NDT, NQS, V_LATE>(c, a.scale, a.softcap, qf, t * TILE_KEYS, M, L, ACC);
+  if (!c.row_ok) return;
+  const int64_t prow = ((int64_t)blockIdx.x * a.nq + head) * a.nseg + seg;
+  if (c.g == 0) {
+    a.part_ml[2 * prow] = M;
+    a.part_ml[2 * prow + 1] = L;
+  }
+  if (M > -INFINITY) {
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt)
+      if (dt * 16 < a.d) *reinterpret_cast<f32x4*>(&a.part_acc[prow * a.d + dt * 16 + 4 * c.g]) = ACC[dt];
+  }
+}
+
 // Folds the segment results of one (token, head) in ascending segment order.
 // One wave per row; lane j owns output columns j, j+64, ...
 __global__ __launch_bounds__(64) void attn_combine_kernel(AttnArgs a) {
@@ -885,7 +1124,9 @@ __global__ __launch_bounds__(64) void attn_combine_kernel(AttnArgs a) {
   const int tok = q_begin + q_off;
   const int pos = k_len - q_len + q_off;
   const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
-  const int seg_begin = lo / (TILE_KEYS * SEG_TILES), seg_end = pos / (TILE_KEYS * SEG_TILES) + 1;
+  // Segments that hold kept first keys come before the window's; those in between were not computed.
+  const int keep_tiles = a.window > 0 ? (a.keep + TILE_KEYS - 1) / TILE_KEYS : 0, tile_lo = lo / TILE_KEYS;
+  const int seg_begin = keep_tiles > 0 ? 0 : lo / (TILE_KEYS * SEG_TILES), seg_end = pos / (TILE_KEYS * SEG_TILES) + 1;
   const int d = a.d;
   float M = -INFINITY, L = 0.f;
   float ACC[4] = {0.f, 0.f, 0.f, 0.f};   // d <= 256
@@ -895,14 +1136,14 @@ __global__ __launch_bounds__(64) void attn_combine_kernel(AttnArgs a) {
     float m[4], l[4], v[4][4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const bool in = seg0 + j < seg_end;
+      const bool in = seg0 + j < seg_end && ((seg0 + j) * SEG_TILES < keep_tiles || (seg0 + j) * SEG_TILES + SEG_TILES > tile_lo);
       const int64_t r = row0 + (in ? seg0 + j : seg_begin);
       m[j] = in ? a.part_ml[2 * r] : -INFINITY;
       l[j] = a.part_ml[2 * r + 1];
     }
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const int64_t r = row0 + (seg0 + j < seg_end ? seg0 + j : seg_begin);
+      const int64_t r = row0 + (m[j] > -INFINITY ? seg0 + j : seg_begin);
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const int col = threadIdx.x + 64 * i;
@@ -921,6 +1162,7 @@ __global__ __launch_bounds__(64) void attn_combine_kernel(AttnArgs a) {
       }
     }
   }
+  if (a.sinks != nullptr && M > -INFINITY) L = L + sink_term(a, head, M);
   const float inv = L > 0.f ? 1.0f / L : 0.f;
   elem_t* orow = a.out + ((int64_t)tok * a.nq + head) * d;
 #pragma unroll
@@ -1112,6 +1354,59 @@ int vk_paged_attention(elem_t* out, const elem_t* q, const elem_t* kc, const ele
   else DECODE_PLAIN(256);
 #undef DECODE_PLAIN
   if (vk_check_launch("attention (decoded rows)")) return 1;
+  attn_combine_kernel<<<dim3(n_items, nq), 64, 0, st>>>(a);
+  return vk_check_launch("attention (combine)");
+}
+
+// The attention with capped scores, kept first keys, a sink and unrounded weights (see "Capped scores" above).
+// mode 0: items of prompt rows; mode 1: items of one decoded token each, with nseg and scratch as vk_paged_attention
+// takes them.  keep > 0 needs a window.  softcap 0: no cap.  sinks: [nq] elements (or floats with sinks_f32) or null.
+int vk_paged_attention_capped(elem_t* out, const elem_t* q, const elem_t* kc, const elem_t* vc, const int32_t* block_table,
+                              int bt_stride, const int32_t* cu_q, const int32_t* k_len, const int32_t* items, int n_items, int mode,
+                              int nseg, float* scratch, int total_tokens, int nq, int nkv, int d, int P, int window, int keep,
+                              float scale, float softcap, const void* sinks, int sinks_f32, hipStream_t st) {
+  (void)total_tokens;
+  VK_REQUIRE(nq > 0 && nkv > 0 && nq % nkv == 0, "attention: %d q heads are not a multiple of %d kv heads", nq, nkv);
+  VK_REQUIRE(d >= 16 && d <= 256 && d % 16 == 0, "attention: head size %d must be a multiple of 16 in 16..256", d);
+  VK_REQUIRE(P >= 8 && (P & (P - 1)) == 0, "attention: page size %d must be a power of two >= 8", P);
+  VK_REQUIRE(window >= 0 && keep >= 0, "attention: window %d and kept keys %d must not be negative", window, keep);
+  VK_REQUIRE(keep == 0 || window > 0, "attention: kept first keys need a window");
+  VK_REQUIRE(scale > 0.f && softcap >= 0.f, "attention: the score scale must be positive and the cap not negative");
+  VK_REQUIRE(mode == 0 || mode == 1, "attention: unknown mode %d", mode);
+  if (n_items <= 0) return 0;
+  AttnArgs a;
+  a.q = q; a.out = out; a.kc = kc; a.vc = vc; a.block_table = block_table; a.cu_q = cu_q; a.k_len = k_len;
+  a.items = items; a.bt_stride = bt_stride; a.nq = nq; a.nkv = nkv; a.d = d; a.P = P; a.window = window;
+  a.nseg = nseg; a.scale_log2 = scale * LOG2E;
+  a.part_ml = nullptr; a.part_acc = nullptr;
+  a.keep = keep; a.scale = scale; a.softcap = softcap; a.sinks = sinks; a.sinks_f32 = sinks_f32;
+  const int G = nq / nkv;
+  if (mode == 0) {
+    const int hpw = G < 4 ? G : 4;
+    VK_REQUIRE((int64_t)n_items * (ITEM_ROWS / 16) < (1ll << 31), "attention: too many prompt items");
+    const dim3 grid(n_items * (ITEM_ROWS / 16), nkv * ((G + hpw - 1) / hpw));
+    VK_REQUIRE(grid.y <= 65535, "attention: too many heads");
+    if (d <= 64) attn_prefill_ext_kernel<64><<<grid, 64 * hpw, 0, st>>>(a, hpw);
+    else if (d <= 128) attn_prefill_ext_kernel<128><<<grid, 64 * hpw, 0, st>>>(a, hpw);
+    else attn_prefill_ext_kernel<256><<<grid, 64 * hpw, 0, st>>>(a, hpw);
+    return vk_check_launch("attention (prompt rows, capped scores)");
+  }
+  VK_REQUIRE(nseg > 0 && nseg <= 65535 && scratch != nullptr, "attention: decode needs nseg in 1..65535 and scratch");
+  a.part_ml = scratch;
+  a.part_acc = scratch + (((int64_t)n_items * nq * nseg * 2 + 3) & ~(int64_t)3);
+  const dim3 grid(n_items, nkv * ((G + 15) / 16), (nseg + PLAIN_WAVES - 1) / PLAIN_WAVES);
+  VK_REQUIRE(grid.y <= 65535 && nq <= 65535, "attention: too many heads");
+  const bool late = (int64_t)grid.x * grid.y * nseg > 1024;
+#define DECODE_EXT(DP)                                                                   \
+  do {                                                                                   \
+    if (late) attn_decode_ext_kernel<DP, true><<<grid, 64 * PLAIN_WAVES, 0, st>>>(a);    \
+    else attn_decode_ext_kernel<DP, false><<<grid, 64 * PLAIN_WAVES, 0, st>>>(a);        \
+  } while (0)
+  if (d <= 64) DECODE_EXT(64);
+  else if (d <= 128) DECODE_EXT(128);
+  else DECODE_EXT(256);
+#undef DECODE_EXT
+  if (vk_check_launch("attention (decoded rows, capped scores)")) return 1;
   attn_combine_kernel<<<dim3(n_items, nq), 64, 0, st>>>(a);
   return vk_check_launch("attention (combine)");
 }

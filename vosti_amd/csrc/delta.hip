@@ -1,0 +1,244 @@
+// The gated delta rule with one decay per head and key channel, and what stands around it: the short causal
+// convolution with its carried inputs, the unit norms, the decays, the recurrence over a state that is carried from
+// step to step in 32-bit, and the gated norm of its read-out.
+//
+// Per head, with the state S [dim, vdim] (rows are key channels), for every token in order:
+//   S <- diag(g) S;  u = beta * (v - S^T k);  S <- S + k u^T;  o = S^T q
+// so that the read-out sees the token's own write.  g = exp(-exp(A_log) * softplus(a + dt_bias)), beta = sigmoid(b).
+// Everything here is 32-bit; the projections that feed it (a, b, the convolutions' inputs) arrive as elements.
+//
+// A sequence's tokens are walked in order by one wave per (sequence, head, block of value columns), so the sums of a
+// token do not depend on how the sequence was cut into steps or on what else is in the batch: the state that a step
+// leaves in memory is the state the next step starts from, bit for bit.
+#include "common.h"
+#include "vec.h"
+
+#define DELTA_MAX_TAPS 16
+
+__device__ __forceinline__ float silu_f(float z) { return z / (1.f + expf(-z)); }
+__device__ __forceinline__ float sigmoid_f(float z) { return 1.f / (1.f + expf(-z)); }
+
+// y[t, c] = silu(sum over j of taps[c, j] * x[t - (K - 1) + j, c]): inputs before the step's first token come from the
+// sequence's carried tail (its last K - 1 inputs, oldest first), or are zero when the sequence starts here.
+__global__ __launch_bounds__(256) void delta_conv_kernel(float* __restrict__ y, const elem_t* __restrict__ x, int64_t ldx,
+                                                         const elem_t* __restrict__ taps, const float* __restrict__ state,
+                                                         int64_t state_stride, int64_t tail_offset, const int32_t* __restrict__ token_seq,
+                                                         const int32_t* __restrict__ cu_q, const int32_t* __restrict__ positions,
+                                                         const int32_t* __restrict__ slots, int C, int K) {
+  const int t = blockIdx.x;
+  const int s = token_seq[t];
+  const int first = cu_q[s], i = t - first;
+  const bool fresh = positions[first] == 0;
+  const float* tail = state + (int64_t)slots[s] * state_stride + tail_offset;
+  for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < C; c += gridDim.y * blockDim.x) {
+    float acc = 0.f;
+    for (int j = 0; j < K; ++j) {
+      const int li = i - (K - 1) + j;
+      float v;
+      if (li >= 0) v = to_f32(x[(int64_t)(first + li) * ldx + c]);
+      else v = fresh ? 0.f : tail[(int64_t)(K - 1 + li) * C + c];
+      acc = acc + to_f32(taps[(int64_t)c * K + j]) * v;
+    }
+    y[(int64_t)t * C + c] = silu_f(acc);
+  }
+}
+
+// The tail after the step: the last K - 1 inputs of the sequence, oldest first.
+__global__ __launch_bounds__(256) void delta_conv_tail_kernel(const elem_t* __restrict__ x, int64_t ldx, float* state,
+                                                              int64_t state_stride, int64_t tail_offset,
+                                                              const int32_t* __restrict__ cu_q, const int32_t* __restrict__ positions,
+                                                              const int32_t* __restrict__ slots, int C, int K) {
+  const int s = blockIdx.x;
+  const int first = cu_q[s], n = cu_q[s + 1] - first;
+  const bool fresh = positions[first] == 0;
+  float* tail = state + (int64_t)slots[s] * state_stride + tail_offset;
+  for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < C; c += gridDim.y * blockDim.x) {
+    float keep[DELTA_MAX_TAPS];
+#pragma unroll
+    for (int r = 0; r < DELTA_MAX_TAPS; ++r) {
+      if (r < K - 1) {
+        const int li = n - (K - 1) + r;
+        keep[r] = li >= 0 ? to_f32(x[(int64_t)(first + li) * ldx + c]) : (fresh ? 0.f : tail[(int64_t)(K - 1 + li) * C + c]);
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < DELTA_MAX_TAPS; ++r)
+      if (r < K - 1) tail[(int64_t)r * C + c] = keep[r];
+  }
+}
+
+// x[t, head, :] <- x / sqrt(sum(x^2) + eps) * scale for `heads` heads of d channels that start at column col0 of rows
+// of length ld.  One wave per (token, head); lane l owns channels l, l + 64, ...
+__global__ __launch_bounds__(64) void delta_unit_kernel(float* x, int64_t ld, int col0, int heads, int d, float eps, float scale) {
+  const int t = blockIdx.x / heads, h = blockIdx.x - t * heads;
+  float* row = x + (int64_t)t * ld + col0 + (int64_t)h * d;
+  float part = 0.f;
+  for (int c = threadIdx.x; c < d; c += 64) part = part + row[c] * row[c];
+  const float r = scale / sqrtf(wave_sum_xor(part) + eps);
+  for (int c = threadIdx.x; c < d; c += 64) row[c] = row[c] * r;
+}
+
+// g[t, h, c] = exp(-exp(A_log[h]) * softplus(a[t, h * d + c] + dt_bias[h * d + c])).
+__global__ __launch_bounds__(256) void delta_decay_kernel(float* __restrict__ g, const elem_t* __restrict__ a, const void* __restrict__ dt_bias,
+                                                          const void* __restrict__ A_log, int w_is_f32, int d, int HD, int64_t numel) {
+  const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= numel) return;
+  const int col = (int)(e % HD);
+  const float z = to_f32(a[e]) + load_weight(dt_bias, w_is_f32, col);
+  const float sp = z > 20.f ? z : log1pf(expf(z));
+  g[e] = expf(-expf(load_weight(A_log, w_is_f32, col / d)) * sp);
+}
+
+// The recurrence.  A wave takes 64 / R value columns of one (sequence, head); a column's state is spread over R
+// neighbouring lanes, lane r of them holding the key channels r, r + R, ... (DR of them at most) in registers.
+// The two sums of a token run over a lane's channels in ascending order and then as a butterfly over the R lanes.
+template <int DR>
+__global__ __launch_bounds__(64) void delta_rule_kernel(float* __restrict__ out, const float* __restrict__ qkv, int64_t ld, int q_col,
+                                                        int k_col, int v_col, const float* __restrict__ decay, const elem_t* __restrict__ b,
+                                                        int64_t ldb, float* state, int64_t state_stride,
+                                                        const int32_t* __restrict__ cu_q, const int32_t* __restrict__ positions,
+                                                        const int32_t* __restrict__ slots, int H, int G, int d, int dv, int R) {
+  const int s = blockIdx.x, h = blockIdx.y;
+  const int lane = threadIdx.x;
+  const int r = lane % R, cols = 64 / R;
+  const int col = blockIdx.z * cols + lane / R;
+  const bool col_ok = col < dv;
+  const int g = h / (H / G);
+  const int first = cu_q[s], n = cu_q[s + 1] - first;
+  const bool fresh = positions[first] == 0;
+  float* S_mem = state + (int64_t)slots[s] * state_stride + (int64_t)h * d * dv;
+  float S[DR];
+#pragma unroll
+  for (int i = 0; i < DR; ++i) {
+    const int row = r + i * R;
+    S[i] = (!fresh && col_ok && row < d) ? S_mem[(int64_t)row * dv + col] : 0.f;
+  }
+  for (int i0 = 0; i0 < n; ++i0) {
+    const int64_t t = first + i0;
+    const float* qrow = qkv + t * ld + q_col + (int64_t)g * d;
+    const float* krow = qkv + t * ld + k_col + (int64_t)g * d;
+    const float* grow = decay + (t * H + h) * d;
+    const float v = col_ok ? qkv[t * ld + v_col + (int64_t)h * dv + col] : 0.f;
+    const float beta = sigmoid_f(to_f32(b[t * ldb + h]));
+    float kk[DR], qq[DR];
+    float dot = 0.f;
+#pragma unroll
+    for (int i = 0; i < DR; ++i) {
+      const int row = r + i * R;
+      const bool ok = row < d;
+      kk[i] = ok ? krow[row] : 0.f;
+      qq[i] = ok ? qrow[row] : 0.f;
+      const float gg = ok ? grow[row] : 1.f;
+      S[i] = S[i] * gg;
+      dot = dot + S[i] * kk[i];
+    }
+    for (int m = 1; m < R; m <<= 1) dot = dot + __shfl_xor(dot, m, VK_WAVE);
+    const float u = beta * (v - dot);
+    float o = 0.f;
+#pragma unroll
+    for (int i = 0; i < DR; ++i) {
+      S[i] = S[i] + kk[i] * u;
+      o = o + S[i] * qq[i];
+    }
+    for (int m = 1; m < R; m <<= 1) o = o + __shfl_xor(o, m, VK_WAVE);
+    if (col_ok && r == 0) out[(t * H + h) * dv + col] = o;
+  }
+#pragma unroll
+  for (int i = 0; i < DR; ++i) {
+    const int row = r + i * R;
+    if (col_ok && row < d) S_mem[(int64_t)row * dv + col] = S[i];
+  }
+}
+
+// y[t, h, :] = o / sqrt(mean(o^2) + eps) * w * sigmoid(gate[t, h, :]), stored as elements.  One wave per (token, head).
+__global__ __launch_bounds__(64) void delta_out_kernel(elem_t* __restrict__ y, const float* __restrict__ o, const elem_t* __restrict__ gate,
+                                                       int64_t ldg, const void* __restrict__ w, int w_is_f32, int H, int dv, float eps) {
+  const int t = blockIdx.x / H, h = blockIdx.x - t * H;
+  const float* row = o + ((int64_t)t * H + h) * dv;
+  float part = 0.f;
+  for (int c = threadIdx.x; c < dv; c += 64) part = part + row[c] * row[c];
+  const float rr = rsqrtf(wave_sum_xor(part) / (float)dv + eps);
+  for (int c = threadIdx.x; c < dv; c += 64) {
+    const float gt = sigmoid_f(to_f32(gate[(int64_t)t * ldg + (int64_t)h * dv + c]));
+    y[((int64_t)t * H + h) * dv + c] = from_f32<elem_t>(((row[c] * rr) * load_weight(w, w_is_f32, c)) * gt);
+  }
+}
+
+extern "C" {
+
+// Lanes that share a value column, for key size d and value size dv: enough that a lane holds 64 channels at most,
+// and more while whole columns' worth of lanes would idle.
+int vk_delta_lanes_per_column(int d, int dv) {
+  int R = 1;
+  while (R < 64 && (d + R - 1) / R > 64) R *= 2;
+  while (R < 64 && 64 / R >= 2 * dv && (d + R - 1) / R > 8) R *= 2;
+  return R;
+}
+
+// y [T, C] floats from the columns x[:, 0:C] of rows of length ldx; then the tails are moved on.
+int vk_delta_conv(float* y, const elem_t* x, int64_t ldx, const elem_t* taps, float* state, int64_t state_stride, int64_t tail_offset,
+                  const int32_t* token_seq, const int32_t* cu_q, const int32_t* positions, const int32_t* slots, int T, int S, int C, int K,
+                  hipStream_t st) {
+  VK_REQUIRE(T >= 0 && S >= 0 && C > 0 && K >= 1 && K <= DELTA_MAX_TAPS + 1, "short convolution: bad sizes T=%d C=%d taps=%d (at most %d)", T, C, K,
+             DELTA_MAX_TAPS + 1);
+  VK_REQUIRE(ldx >= C && tail_offset >= 0 && state_stride >= tail_offset + (int64_t)(K - 1) * C, "short convolution: the state does not hold the tails");
+  if (T == 0 || S == 0) return 0;
+  const int by = (C + 255) / 256 < 64 ? (C + 255) / 256 : 64;
+  delta_conv_kernel<<<dim3(T, by), 256, 0, st>>>(y, x, ldx, taps, state, state_stride, tail_offset, token_seq, cu_q, positions, slots, C, K);
+  if (vk_check_launch("short convolution")) return 1;
+  if (K > 1) {
+    delta_conv_tail_kernel<<<dim3(S, by), 256, 0, st>>>(x, ldx, state, state_stride, tail_offset, cu_q, positions, slots, C, K);
+    return vk_check_launch("short convolution (tails)");
+  }
+  return 0;
+}
+
+int vk_delta_unit(float* x, int64_t ld, int col0, int T, int heads, int d, float eps, float scale, hipStream_t st) {
+  VK_REQUIRE(T >= 0 && heads > 0 && d > 0 && ld >= col0 + (int64_t)heads * d, "unit norm: bad sizes");
+  if (T == 0) return 0;
+  VK_REQUIRE((int64_t)T * heads < (1ll << 31), "unit norm: too many rows");
+  delta_unit_kernel<<<T * heads, 64, 0, st>>>(x, ld, col0, heads, d, eps, scale);
+  return vk_check_launch("unit norm");
+}
+
+int vk_delta_decay(float* g, const elem_t* a, const void* dt_bias, const void* A_log, int w_is_f32, int T, int H, int d, hipStream_t st) {
+  VK_REQUIRE(T >= 0 && H > 0 && d > 0, "decay: bad sizes");
+  const int64_t numel = (int64_t)T * H * d;
+  if (numel == 0) return 0;
+  delta_decay_kernel<<<(unsigned)((numel + 255) / 256), 256, 0, st>>>(g, a, dt_bias, A_log, w_is_f32, d, H * d, numel);
+  return vk_check_launch("decay");
+}
+
+// out [T, H, dv] floats.  qkv: float rows of length ld with q (G heads of d) at q_col, k at k_col, v (H heads of dv) at
+// v_col; decay [T, H, d] floats; b: elements, beta's pre-activation of head h at b[t * ldb + h].  state: per slot,
+// the H states [d, dv] at its start.
+int vk_delta_rule(float* out, const float* qkv, int64_t ld, int q_col, int k_col, int v_col, const float* decay, const elem_t* b, int64_t ldb,
+                  float* state, int64_t state_stride, const int32_t* cu_q, const int32_t* positions, const int32_t* slots, int S, int H, int G,
+                  int d, int dv, hipStream_t st) {
+  VK_REQUIRE(S >= 0 && H > 0 && G > 0 && H % G == 0 && d > 0 && dv > 0, "delta rule: bad sizes H=%d G=%d d=%d dv=%d", H, G, d, dv);
+  VK_REQUIRE(d <= 4096, "delta rule: key size %d exceeds 4096", d);
+  VK_REQUIRE(state_stride >= (int64_t)H * d * dv, "delta rule: the state is too small");
+  if (S == 0) return 0;
+  const int R = vk_delta_lanes_per_column(d, dv);
+  const int per_lane = (d + R - 1) / R, cols = 64 / R;
+  const dim3 grid(S, H, (dv + cols - 1) / cols);
+  VK_REQUIRE(grid.y <= 65535 && grid.z <= 65535, "delta rule: too many heads or columns");
+#define RULE(DR) delta_rule_kernel<DR><<<grid, 64, 0, st>>>(out, qkv, ld, q_col, k_col, v_col, decay, b, ldb, state, state_stride, cu_q, positions, slots, H, G, d, dv, R)
+  if (per_lane <= 8) RULE(8);
+  else if (per_lane <= 16) RULE(16);
+  else if (per_lane <= 32) RULE(32);
+  else RULE(64);
+#undef RULE
+  return vk_check_launch("delta rule");
+}
+
+int vk_delta_out(elem_t* y, const float* o, const elem_t* gate, int64_t ldg, const void* w, int w_is_f32, int T, int H, int dv, float eps,
+                 hipStream_t st) {
+  VK_REQUIRE(T >= 0 && H > 0 && dv > 0 && ldg >= (int64_t)H * dv, "delta read-out: bad sizes");
+  if (T == 0) return 0;
+  VK_REQUIRE((int64_t)T * H < (1ll << 31), "delta read-out: too many rows");
+  delta_out_kernel<<<T * H, 64, 0, st>>>(y, o, gate, ldg, w, w_is_f32, H, dv, eps);
+  return vk_check_launch("delta read-out");
+}
+
+}  // extern "C"

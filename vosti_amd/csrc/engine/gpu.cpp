@@ -2,6 +2,7 @@
 
 #include <dlfcn.h>
 
+#include <algorithm>
 #include <sstream>
 
 namespace vosti {
@@ -97,9 +98,23 @@ struct Kernels::Fn {
   int64_t (*attn_scratch_floats)(int, int, int, int);
   int (*attn_segment_keys)();
   int (*attn_item_rows)();
+  int (*embed_sinusoid)(P, CP, CP, CP, CP, int, int, int, hipStream_t);
+  int (*stream_norm)(P, CP, int, CP, int, int, int, float, float, hipStream_t);
+  int (*stream_norm_add)(P, CP, CP, CP, int, int, int, float, float, float, hipStream_t);
+  int (*stream_mix)(P, CP, int64_t, CP, int, int, int64_t, hipStream_t);
+  int (*gather_rows_f32)(P, CP, CP, int, int, hipStream_t);
+  int (*softcap)(P, float, int64_t, hipStream_t);
+  int (*qkv_post_bias)(CP, int64_t, P, P, P, CP, CP, int, CP, CP, int, CP, CP, int, int, int, int, int, float, CP, hipStream_t);
+  int (*paged_attention_capped)(P, CP, CP, CP, CP, int, CP, CP, CP, int, int, int, P, int, int, int, int, int, int, int, float, float, CP, int,
+                                hipStream_t);
+  int (*delta_conv)(P, CP, int64_t, CP, P, int64_t, int64_t, CP, CP, CP, CP, int, int, int, int, hipStream_t);
+  int (*delta_unit)(P, int64_t, int, int, int, int, float, float, hipStream_t);
+  int (*delta_decay)(P, CP, CP, CP, int, int, int, int, hipStream_t);
+  int (*delta_rule)(P, CP, int64_t, int, int, int, CP, CP, int64_t, P, int64_t, CP, CP, CP, int, int, int, int, int, hipStream_t);
+  int (*delta_out)(P, CP, CP, int64_t, CP, int, int, int, int, float, hipStream_t);
 };
 
-static constexpr int KERNEL_ABI = 13;
+static constexpr int KERNEL_ABI = 14;
 
 Kernels::Kernels(const std::string& lib_dir, const std::string& name) : name_(name), fn_(new Fn) {
   if (name == "bf16") dtype_ = DType::BF16;
@@ -125,6 +140,11 @@ Kernels::Kernels(const std::string& lib_dir, const std::string& name) : name_(na
   VK(qkv_post, "vk_qkv_post"); VK(paged_attention, "vk_paged_attention"); VK(sample, "vk_sample");
   VK(sample_scratch_words, "vk_sample_scratch_words"); VK(attn_scratch_floats, "vk_attn_scratch_floats");
   VK(attn_segment_keys, "vk_attn_segment_keys"); VK(attn_item_rows, "vk_attn_item_rows");
+  VK(embed_sinusoid, "vk_embed_sinusoid"); VK(stream_norm, "vk_stream_norm"); VK(stream_norm_add, "vk_stream_norm_add");
+  VK(stream_mix, "vk_stream_mix"); VK(gather_rows_f32, "vk_gather_rows_f32"); VK(softcap, "vk_softcap");
+  VK(qkv_post_bias, "vk_qkv_post_bias"); VK(paged_attention_capped, "vk_paged_attention_capped");
+  VK(delta_conv, "vk_delta_conv"); VK(delta_unit, "vk_delta_unit"); VK(delta_decay, "vk_delta_decay"); VK(delta_rule, "vk_delta_rule");
+  VK(delta_out, "vk_delta_out");
 #undef VK
   segment_keys_ = fn_->attn_segment_keys();
   item_rows_ = fn_->attn_item_rows();
@@ -210,12 +230,13 @@ Tensor Kernels::swiglu(const Tensor& gate_up) {
 }
 
 Tensor Kernels::gather_rows(const Tensor& x, const Tensor& rows) {
-  expect(x, "rows' source", dtype_);
+  if (x.dtype != DType::F32) expect(x, "rows' source", dtype_);
   if (x.shape.size() != 2) throw EngineError("gather_rows: source is " + x.describe());
   const int64_t R = rows.numel();
   expect(rows, "row numbers", DType::I32, {R});
-  Tensor out = empty({R, x.dim(1)});
-  call(fn_->gather_rows(out.data, x.data, rows.data, (int)R, (int)x.dim(1), stream));
+  Tensor out = empty({R, x.dim(1)}, x.dtype);
+  if (x.dtype == DType::F32 && dtype_ != DType::F32) call(fn_->gather_rows_f32(out.data, x.data, rows.data, (int)R, (int)x.dim(1), stream));
+  else call(fn_->gather_rows(out.data, x.data, rows.data, (int)R, (int)x.dim(1), stream));
   return out;
 }
 
@@ -380,6 +401,193 @@ void Kernels::paged_attention(Tensor& out, const Tensor& q, const Tensor& k_cach
   call(fn_->paged_attention(out.data, q.data, k_cache.data, v_cache.data, block_table.data, (int)W, cu_q.data, k_len.data,
                             items.data, (int)n_items, mode, nseg, sp, (int)T, (int)nq, (int)nkv, (int)d, (int)P, window, scale,
                             stream));
+}
+
+// ------------------------------------------------------------------------- the 32-bit residual stream
+Tensor Kernels::embed_sinusoid(const Tensor& table, const Tensor& ids, const Tensor& positions, const Tensor& inv_freq) {
+  expect(table, "embedding table", dtype_);
+  if (table.shape.size() != 2) throw EngineError("embedding table is " + table.describe());
+  const int64_t V = table.dim(0), H = table.dim(1), T = ids.numel();
+  expect(ids, "ids", DType::I32, {T});
+  expect(positions, "positions", DType::I32, {T});
+  expect(inv_freq, "inverse frequencies", DType::F32, {H / 2});
+  Tensor out = empty({T, H}, DType::F32);
+  call(fn_->embed_sinusoid(out.data, table.data, ids.data, positions.data, inv_freq.data, (int)T, (int)H, (int)V, stream));
+  return out;
+}
+
+Tensor Kernels::stream_norm(const Tensor& x, const Tensor& w, float eps, float offset) {
+  if (x.dtype != DType::F32) expect(x, "norm input", dtype_);
+  if (x.shape.empty()) throw EngineError("norm input is " + x.describe());
+  const int64_t H = x.dim(-1), rows = H ? x.numel() / H : 0;
+  const int wf = norm_weight(w, "norm weight", H);
+  Tensor out = empty(x.shape);
+  call(fn_->stream_norm(out.data, x.data, x.dtype == DType::F32 ? 1 : 0, w.data, wf, (int)rows, (int)H, eps, offset, stream));
+  return out;
+}
+
+void Kernels::stream_norm_add(Tensor& out, const Tensor& base, const Tensor& y, const Tensor& w, float eps, float offset, float mult) {
+  expect(y, "norm input", dtype_);
+  if (y.shape.size() != 2) throw EngineError("norm input is " + y.describe());
+  expect(base, "stream", DType::F32, y.shape);
+  expect(out, "stream", DType::F32, y.shape);
+  const int wf = norm_weight(w, "norm weight", y.dim(1));
+  call(fn_->stream_norm_add(out.data, base.data, y.data, w.data, wf, (int)y.dim(0), (int)y.dim(1), eps, offset, mult, stream));
+}
+
+Tensor Kernels::stream_mix(const Tensor& states, const Tensor& coef, int n) {
+  expect(states, "stream states", DType::F32);
+  if (states.shape.size() < 2 || n <= 0 || n > states.dim(0)) throw EngineError("stream mix: " + std::to_string(n) + " of " + states.describe());
+  const int cf = norm_weight(coef, "mixing weights", n);
+  std::vector<int64_t> shape(states.shape.begin() + 1, states.shape.end());
+  Tensor out = empty(shape, DType::F32);
+  const int64_t numel = out.numel();
+  call(fn_->stream_mix(out.data, states.data, numel, coef.data, cf, n, numel, stream));
+  return out;
+}
+
+void Kernels::softcap(Tensor& x, float cap) {
+  expect(x, "values to cap", dtype_);
+  call(fn_->softcap(x.data, cap, x.numel(), stream));
+}
+
+Tensor Kernels::gemm_columns(const Tensor& act, int64_t first, const Tensor& w) {
+  expect(act, "activation", dtype_);
+  expect(w, "weight", dtype_);
+  if (act.shape.size() != 2 || w.shape.size() != 2 || first < 0 || first + w.dim(1) > act.dim(1))
+    throw EngineError("gemm: columns " + std::to_string(first) + ".. of " + act.describe() + " do not fit weight " + w.describe());
+  const int vec = 16 / dtype_bytes(dtype_);
+  if (first % vec || act.dim(1) % vec) throw EngineError("gemm: columns must start on a 16-byte boundary");
+  const int64_t M = act.dim(0), K = w.dim(1), N = w.dim(0);
+  Tensor out = empty({M, N});
+  call(fn_->gemm(out.data, static_cast<const char*>(act.data) + (size_t)first * dtype_bytes(dtype_), w.data, (int)M, (int)N, (int)K, act.dim(1), N,
+                 0, stream));
+  return out;
+}
+
+Tensor Kernels::qkv_post_bias(const Tensor& qkv, int nq, int nkv, int d, const Tensor* k_cache, const Tensor* v_cache, int page_size,
+                              const Tensor* slots, const Tensor& bias) {
+  expect(qkv, "qkv", dtype_);
+  const int64_t W = (int64_t)(nq + 2 * nkv) * d;
+  if (qkv.shape.size() != 2 || qkv.dim(1) != W) throw EngineError("qkv_post: rows are " + qkv.describe() + ", expected width " + std::to_string(W));
+  expect(bias, "qkv bias", dtype_, {W});
+  const int64_t T = qkv.dim(0);
+  Tensor q_out;
+  if (nq) q_out = empty({T, nq, d});
+  if (nkv) {
+    if (!k_cache || !v_cache || !slots) throw EngineError("qkv_post: a store needs both caches and slots");
+    if (k_cache->shape.size() != 4) throw EngineError("k cache is " + k_cache->describe());
+    const int64_t pages = k_cache->dim(0);
+    expect(*k_cache, "k cache", dtype_, {pages, nkv, page_size, d});
+    expect(*v_cache, "v cache", dtype_, {pages, nkv, d, page_size});
+    expect(*slots, "slots", DType::I32, {T});
+  }
+  call(fn_->qkv_post_bias(qkv.data, W, nq ? q_out.data : nullptr, nkv ? k_cache->data : nullptr, nkv ? v_cache->data : nullptr, nullptr, nullptr, 0,
+                          nullptr, nullptr, 0, nullptr, nkv ? slots->data : nullptr, (int)T, nq, nkv, d, page_size, 0.f, bias.data, stream));
+  return q_out;
+}
+
+void Kernels::paged_attention_capped(Tensor& out, const Tensor& q, const Tensor& k_cache, const Tensor& v_cache, const Tensor& block_table,
+                                     const Tensor& cu_q, const Tensor& k_len, const Tensor& items, int mode, float scale, int window, int keep,
+                                     float softcap, const Tensor* sinks, int max_k_len, int nseg, const Tensor* scratch) {
+  expect(q, "q", dtype_);
+  expect(block_table, "block table", DType::I32);
+  if (q.shape.size() != 3 || k_cache.shape.size() != 4 || block_table.shape.size() != 2)
+    throw EngineError("attention: q " + q.describe() + ", k cache " + k_cache.describe() + ", block table " + block_table.describe());
+  const int64_t T = q.dim(0), nq = q.dim(1), d = q.dim(2), pages = k_cache.dim(0), nkv = k_cache.dim(1), P = k_cache.dim(2);
+  const int64_t S = block_table.dim(0), W = block_table.dim(1);
+  expect(k_cache, "k cache", dtype_, {pages, nkv, P, d});
+  expect(v_cache, "v cache", dtype_, {pages, nkv, d, P});
+  expect(cu_q, "cu_q", DType::I32, {S + 1});
+  expect(k_len, "k_len", DType::I32, {S});
+  expect(out, "attention output", dtype_, q.shape);
+  if (items.shape.size() != 2 || items.dim(1) != 2) throw EngineError("attention: items are " + items.describe());
+  expect(items, "items", DType::I32);
+  if (mode != 0 && mode != 1) throw EngineError("attention with capped scores: mode " + std::to_string(mode));
+  if (W * P < max_k_len)
+    throw EngineError("attention: a block table of " + std::to_string(W) + " pages of " + std::to_string(P) + " does not cover " +
+                      std::to_string(max_k_len) + " keys");
+  int sf = 0;
+  if (sinks) sf = norm_weight(*sinks, "attention sinks", nq);
+  void* sp = nullptr;
+  const int64_t n_items = items.dim(0);
+  if (mode == 1) {
+    if (nseg < (max_k_len + segment_keys_ - 1) / segment_keys_)
+      throw EngineError("attention: " + std::to_string(nseg) + " segments do not cover " + std::to_string(max_k_len) + " keys");
+    const int64_t need = attn_scratch_floats((int)n_items, (int)nq, (int)d, nseg);
+    if (!scratch || scratch->dtype != DType::F32 || scratch->numel() < need)
+      throw EngineError("attention: scratch of " + std::to_string(need) + " floats needed");
+    sp = scratch->data;
+  }
+  call(fn_->paged_attention_capped(out.data, q.data, k_cache.data, v_cache.data, block_table.data, (int)W, cu_q.data, k_len.data, items.data,
+                                   (int)n_items, mode, nseg, sp, (int)T, (int)nq, (int)nkv, (int)d, (int)P, window, keep, scale, softcap,
+                                   sinks ? sinks->data : nullptr, sf, stream));
+}
+
+// ------------------------------------------------------------------------------------- the delta rule
+Tensor Kernels::delta_conv(const Tensor& x, const Tensor& taps, Tensor& state, int64_t tail_offset, const Tensor& token_seq, const Tensor& cu_q,
+                           const Tensor& positions, const Tensor& slots) {
+  expect(x, "convolution input", dtype_);
+  expect(taps, "convolution taps", dtype_);
+  expect(state, "state", DType::F32);
+  if (x.shape.size() != 2 || taps.shape.size() != 2 || state.shape.size() != 2 || taps.dim(0) > x.dim(1))
+    throw EngineError("short convolution: input " + x.describe() + ", taps " + taps.describe() + ", state " + state.describe());
+  const int64_t T = x.dim(0), C = taps.dim(0), K = taps.dim(1), S = slots.numel();
+  expect(token_seq, "token sequences", DType::I32, {T});
+  expect(positions, "positions", DType::I32, {T});
+  expect(cu_q, "cu_q", DType::I32, {S + 1});
+  expect(slots, "state slots", DType::I32, {S});
+  Tensor y = empty({T, C}, DType::F32);
+  call(fn_->delta_conv(y.data, x.data, x.dim(1), taps.data, state.data, state.dim(1), tail_offset, token_seq.data, cu_q.data, positions.data,
+                       slots.data, (int)T, (int)S, (int)C, (int)K, stream));
+  return y;
+}
+
+void Kernels::delta_unit(Tensor& x, int64_t col0, int heads, int d, float eps, float scale) {
+  expect(x, "unit norm input", DType::F32);
+  if (x.shape.size() != 2) throw EngineError("unit norm input is " + x.describe());
+  call(fn_->delta_unit(x.data, x.dim(1), (int)col0, (int)x.dim(0), heads, d, eps, scale, stream));
+}
+
+Tensor Kernels::delta_decay(const Tensor& a, const Tensor& dt_bias, const Tensor& A_log, int H, int d) {
+  expect(a, "decay input", dtype_);
+  if (a.shape.size() != 2 || a.dim(1) != (int64_t)H * d) throw EngineError("decay input is " + a.describe());
+  const int wf = norm_weight(dt_bias, "dt_bias", (int64_t)H * d);
+  if (norm_weight(A_log, "A_log", H) != wf) throw EngineError("decay: dt_bias and A_log must have one type");
+  Tensor g = empty({a.dim(0), H, d}, DType::F32);
+  call(fn_->delta_decay(g.data, a.data, dt_bias.data, A_log.data, wf, (int)a.dim(0), H, d, stream));
+  return g;
+}
+
+Tensor Kernels::delta_rule(const Tensor& qkv, int q_col, int k_col, int v_col, const Tensor& decay, const Tensor& b, int64_t b_col, Tensor& state,
+                           const Tensor& cu_q, const Tensor& positions, const Tensor& slots, int H, int G, int d, int dv) {
+  expect(qkv, "delta rule input", DType::F32);
+  expect(b, "beta input", dtype_);
+  expect(state, "state", DType::F32);
+  if (qkv.shape.size() != 2 || b.shape.size() != 2 || state.shape.size() != 2 || b.dim(0) != qkv.dim(0) || b_col + H > b.dim(1) ||
+      std::max(q_col, k_col) + (int64_t)G * d > qkv.dim(1) || v_col + (int64_t)H * dv > qkv.dim(1))
+    throw EngineError("delta rule: input " + qkv.describe() + ", beta " + b.describe() + ", state " + state.describe());
+  const int64_t T = qkv.dim(0), S = slots.numel();
+  expect(decay, "decay", DType::F32, {T, H, d});
+  expect(positions, "positions", DType::I32, {T});
+  expect(cu_q, "cu_q", DType::I32, {S + 1});
+  expect(slots, "state slots", DType::I32, {S});
+  Tensor out = empty({T, H, dv}, DType::F32);
+  call(fn_->delta_rule(out.data, qkv.data, qkv.dim(1), q_col, k_col, v_col, decay.data,
+                       static_cast<const char*>(b.data) + (size_t)b_col * dtype_bytes(dtype_), b.dim(1), state.data, state.dim(1), cu_q.data,
+                       positions.data, slots.data, (int)S, H, G, d, dv, stream));
+  return out;
+}
+
+Tensor Kernels::delta_out(const Tensor& o, const Tensor& gate, const Tensor& w, int H, int dv, float eps) {
+  expect(o, "delta read-out", DType::F32);
+  expect(gate, "gate", dtype_);
+  if (o.shape.size() != 3 || o.dim(1) != H || o.dim(2) != dv || gate.shape.size() != 2 || gate.dim(0) != o.dim(0) || gate.dim(1) != (int64_t)H * dv)
+    throw EngineError("delta read-out: " + o.describe() + " with gate " + gate.describe());
+  const int wf = norm_weight(w, "read-out norm weight", dv);
+  Tensor y = empty({o.dim(0), (int64_t)H * dv});
+  call(fn_->delta_out(y.data, o.data, gate.data, gate.dim(1), w.data, wf, (int)o.dim(0), H, dv, eps, stream));
+  return y;
 }
 
 int Kernels::sample_scratch_words(int rows) const { return fn_->sample_scratch_words(rows); }

@@ -135,6 +135,34 @@ class Kernels {
   // Token ids per row: the largest logit, or a draw at temps[r] > 0 with the uniform number unis[r].
   void sample(Tensor& out, const Tensor& logits, const Tensor* temps, const Tensor* unis, Tensor& scratch);
   int sample_scratch_words(int rows) const;
+  // ---- a residual stream in 32-bit whatever the element type (stream.hip)
+  // table[ids] + sinusoidal positions (entry 2i: sin(p f[i]), 2i + 1: cos(p f[i])) as floats [T, width].
+  Tensor embed_sinusoid(const Tensor& table, const Tensor& ids, const Tensor& positions, const Tensor& inv_freq);
+  // x (floats or elements) * rsqrt(mean(x^2) + eps) * (offset + w), as elements.
+  Tensor stream_norm(const Tensor& x, const Tensor& w, float eps, float offset);
+  // out = base + mult * norm(y), floats; out may be base.
+  void stream_norm_add(Tensor& out, const Tensor& base, const Tensor& y, const Tensor& w, float eps, float offset, float mult);
+  // out = sum over j < n of coef[j] * states[j]; states [>= n, ...] floats.
+  Tensor stream_mix(const Tensor& states, const Tensor& coef, int n);
+  void softcap(Tensor& x, float cap);          // x <- cap * tanh(x / cap)
+  // gemm on the columns [first, first + w.dim(1)) of act.
+  Tensor gemm_columns(const Tensor& act, int64_t first, const Tensor& w);
+  // qkv_post with a bias [(nq + 2 nkv) d] added to the rows first.
+  Tensor qkv_post_bias(const Tensor& qkv, int nq, int nkv, int d, const Tensor* k_cache, const Tensor* v_cache, int page_size,
+                       const Tensor* slots, const Tensor& bias);
+  // Attention with capped scores, kept first keys, a sink per head and unrounded weights (attention.hip).
+  void paged_attention_capped(Tensor& out, const Tensor& q, const Tensor& k_cache, const Tensor& v_cache, const Tensor& block_table,
+                              const Tensor& cu_q, const Tensor& k_len, const Tensor& items, int mode, float scale, int window, int keep,
+                              float softcap, const Tensor* sinks, int max_k_len, int nseg, const Tensor* scratch);
+  // ---- the gated delta rule with a decay per key channel (delta.hip)
+  // silu(short causal convolution) of the first taps.dim(0) columns of x, floats [T, C]; the state's tails move on.
+  Tensor delta_conv(const Tensor& x, const Tensor& taps, Tensor& state, int64_t tail_offset, const Tensor& token_seq, const Tensor& cu_q,
+                    const Tensor& positions, const Tensor& slots);
+  void delta_unit(Tensor& x, int64_t col0, int heads, int d, float eps, float scale);
+  Tensor delta_decay(const Tensor& a, const Tensor& dt_bias, const Tensor& A_log, int H, int d);
+  Tensor delta_rule(const Tensor& qkv, int q_col, int k_col, int v_col, const Tensor& decay, const Tensor& b, int64_t b_col, Tensor& state,
+                    const Tensor& cu_q, const Tensor& positions, const Tensor& slots, int H, int G, int d, int dv);
+  Tensor delta_out(const Tensor& o, const Tensor& gate, const Tensor& w, int H, int dv, float eps);
   int segment_keys() const { return segment_keys_; }
   int item_rows() const { return item_rows_; }
 

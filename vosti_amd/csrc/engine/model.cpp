@@ -39,6 +39,14 @@ std::string join(const std::vector<std::string>& v, const char* sep) {
   return s;
 }
 
+// Whether a stored shape is what a parameter declares; a declared -1 takes any size.
+bool shape_fits(const std::vector<int64_t>& stored, const std::vector<int64_t>& declared) {
+  if (stored.size() != declared.size()) return false;
+  for (size_t i = 0; i < stored.size(); ++i)
+    if (declared[i] >= 0 && declared[i] != stored[i]) return false;
+  return true;
+}
+
 bool is_float_type(const std::string& t) { return t == "F64" || t == "F32" || t == "F16" || t == "BF16"; }
 bool is_int_type(const std::string& t) { return t == "I64" || t == "I32" || t == "I16" || t == "I8" || t == "U8" || t == "BOOL"; }
 
@@ -174,7 +182,7 @@ void DecoderModel::load_weights(const Checkpoint& ckpt) {
     auto it = stored.find(e.first);
     if (it == stored.end()) {
       missing.push_back(e.first);
-    } else if (it->second.shape != e.second.decl.shape) {
+    } else if (!shape_fits(it->second.shape, e.second.decl.shape)) {
       wrong.push_back(e.first + ": file has " + shape_text(it->second.shape) + ", model needs " + shape_text(e.second.decl.shape));
     } else if (!is_float_type(it->second.dtype) && !is_int_type(it->second.dtype)) {
       wrong.push_back(e.first + ": unsupported stored type " + it->second.dtype);
@@ -277,6 +285,8 @@ void DecoderModel::random_weights(uint64_t seed) {
     Tensor t;
     t.dtype = kernels_.dtype();
     t.shape = d.shape;
+    for (int64_t& s : t.shape)
+      if (s < 0) s = d.free_size;
     t.owner = std::make_shared<DeviceBuffer>(t.bytes());
     t.data = t.owner->data();
     // As the kernel takes them: a normal value is a sum of four 16-bit uniforms times std * sqrt(3) / 65536.
@@ -308,7 +318,7 @@ std::vector<CacheNeed> DecoderModel::cache_needs() {
 Tensor DecoderModel::forward(const Tensor& ids, StepContext& ctx, std::vector<CacheEntry>& caches, const Tensor& want_rows) {
   if (!loaded_) throw EngineError("the model has no weights yet");
   if (caches.size() != spec_.schedule.size()) throw EngineError("one cache entry per schedule entry is needed");
-  Tensor hidden = embedding_->forward(ids), residual;
+  Tensor hidden = embedding_->forward(ids, ctx), residual;
   for (size_t i = 0; i < spec_.schedule.size(); ++i) {
     auto hr = layers_[spec_.schedule[i].layer]->forward(hidden, residual, ctx, caches[i]);
     hidden = hr.first;

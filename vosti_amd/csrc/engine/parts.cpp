@@ -4,6 +4,7 @@
 
 #include <dlfcn.h>
 
+#include <algorithm>
 #include <cmath>
 #include <mutex>
 
@@ -83,6 +84,11 @@ std::pair<Tensor, Tensor> PositionEncoding::apply(const Tensor& q, const Tensor&
   return {rotate(q), k.data ? rotate(k) : Tensor()};
 }
 
+void Norm::forward_scaled_add(const Tensor& y, const Tensor& base, Tensor& out, float mult) {
+  (void)y; (void)base; (void)out; (void)mult;
+  throw EngineError("this norm kind cannot add its scaled output to a 32-bit residual stream");
+}
+
 std::unique_ptr<Part> build_any_part(const std::string& category, const PartSpec& spec, Kernels& k) {
   auto it = part_registry().find({category, spec.kind});
   if (it == part_registry().end()) throw ConfigError("no " + category + " part of kind '" + spec.kind + "' in the native engine");
@@ -95,7 +101,7 @@ std::unique_ptr<Block> build_block(const LayerSpec& spec, Kernels& k) {
   std::map<std::string, std::unique_ptr<Norm>> norms;
   for (const auto& n : spec.norms) norms[n.first] = build_part<Norm>("norm", *n.second, k);
   return it->second(k, build_part<Mixer>("mixer", *spec.mixer, k), build_part<FeedForward>("feed_forward", *spec.feed_forward, k),
-                    std::move(norms));
+                    std::move(norms), spec.block_numbers);
 }
 
 namespace {
@@ -127,6 +133,59 @@ Tensor stack_rows(const std::vector<Tensor>& pieces) {
   return out;
 }
 
+Tensor zero_weight(std::vector<int64_t> shape, DType t) {
+  Tensor out;
+  out.dtype = t;
+  out.shape = std::move(shape);
+  out.owner = std::make_shared<DeviceBuffer>(out.bytes());
+  out.data = out.owner->data();
+  hip_check(hipMemset(out.data, 0, out.bytes()), "clearing a weight");
+  return out;
+}
+
+// w [rows, cols] in the upper left corner of a zero matrix [rows_to, cols_to].
+Tensor pad_matrix(const Tensor& w, int64_t rows_to, int64_t cols_to) {
+  if (w.shape.size() != 2 || rows_to < w.dim(0) || cols_to < w.dim(1)) throw EngineError("a weight cannot be padded to a smaller size");
+  if (rows_to == w.dim(0) && cols_to == w.dim(1)) return w;
+  Tensor out = zero_weight({rows_to, cols_to}, w.dtype);
+  const size_t e = (size_t)dtype_bytes(w.dtype);
+  if (w.numel())
+    hip_check(hipMemcpy2D(out.data, (size_t)cols_to * e, w.data, (size_t)w.dim(1) * e, (size_t)w.dim(1) * e, (size_t)w.dim(0), hipMemcpyDeviceToDevice),
+              "padding a weight");
+  return out;
+}
+
+// The rows of w [n * size, cols] as n blocks of size_to rows each, the new rows zero: a head's outputs padded.
+Tensor pad_row_blocks(const Tensor& w, int64_t n, int64_t size, int64_t size_to) {
+  const bool vec = w.shape.size() == 1;
+  const Tensor m = vec ? w.view({w.dim(0), 1}) : w;
+  if (m.shape.size() != 2 || m.dim(0) != n * size || size_to < size) throw EngineError("a weight of " + w.describe() + " is not " + std::to_string(n) + " blocks of " + std::to_string(size) + " rows");
+  if (size_to == size) return w;
+  Tensor out = zero_weight({n * size_to, m.dim(1)}, w.dtype);
+  const size_t row = (size_t)m.dim(1) * dtype_bytes(w.dtype);
+  for (int64_t b = 0; b < n; ++b)
+    hip_check(hipMemcpy(static_cast<char*>(out.data) + (size_t)(b * size_to) * row, static_cast<const char*>(m.data) + (size_t)(b * size) * row,
+                        (size_t)size * row, hipMemcpyDeviceToDevice),
+              "padding a weight");
+  return vec ? out.view({n * size_to}) : out;
+}
+
+// The columns of w [rows, n * size] as n blocks of size_to columns each, the new columns zero: a head's inputs padded.
+Tensor pad_column_blocks(const Tensor& w, int64_t n, int64_t size, int64_t size_to) {
+  if (w.shape.size() != 2 || w.dim(1) != n * size || size_to < size) throw EngineError("a weight of " + w.describe() + " is not " + std::to_string(n) + " blocks of " + std::to_string(size) + " columns");
+  if (size_to == size) return w;
+  Tensor out = zero_weight({w.dim(0), n * size_to}, w.dtype);
+  const size_t e = (size_t)dtype_bytes(w.dtype);
+  for (int64_t b = 0; b < n; ++b)
+    hip_check(hipMemcpy2D(static_cast<char*>(out.data) + (size_t)(b * size_to) * e, (size_t)(n * size_to) * e,
+                          static_cast<const char*>(w.data) + (size_t)(b * size) * e, (size_t)(n * size) * e, (size_t)size * e, (size_t)w.dim(0),
+                          hipMemcpyDeviceToDevice),
+              "padding a weight");
+  return out;
+}
+
+int64_t round_up(int64_t n, int64_t to) { return (n + to - 1) / to * to; }
+
 // h[t] = E[ids[t]], a row copy without scale (src/exec/dense_swiglu_model.rs:271-273).
 class TokenEmbedding : public Embedding {
  public:
@@ -140,21 +199,61 @@ class TokenEmbedding : public Embedding {
   Tensor weight_;
 };
 
+// h[t] = E[ids[t]] + s(position of t), where s has sin(p * base^(-2i / width)) at entry 2i and the cosine of the same
+// angle at entry 2i + 1.  The result is the residual stream in 32-bit, whatever the element type.  The frequencies are
+// the 32-bit numbers that every host of these kernels computes for a rotation of the same base and width.
+class SinusoidEmbedding : public Embedding {
+ public:
+  SinusoidEmbedding(const PartSpec& s, Kernels& k)
+      : Embedding(k), vocab_(s.integer("vocab_size")), hidden_(s.integer("hidden_size")), base_(s.number("base")) {
+    if (hidden_ % 2) throw ConfigError("sinusoidal positions need an even width, not " + std::to_string(hidden_));
+  }
+  std::vector<ParamDecl> params() const override { return {{"weight", {vocab_, hidden_}}}; }
+  void load(std::map<std::string, Tensor>& t) override {
+    weight_ = need(t, "weight");
+    std::vector<float> inv((size_t)hidden_ / 2);
+    rotary_inverse_frequencies(base_, (int)hidden_, inv.data());
+    inv_freq_ = zero_weight({hidden_ / 2}, DType::F32);
+    hip_check(hipMemcpy(inv_freq_.data, inv.data(), inv.size() * sizeof(float), hipMemcpyHostToDevice), "position frequencies");
+  }
+  Tensor forward(const Tensor&) override { throw EngineError("an embedding with positions needs the step's positions"); }
+  Tensor forward(const Tensor& ids, StepContext& ctx) override { return kernels.embed_sinusoid(weight_, ids, ctx.positions, inv_freq_); }
+
+ private:
+  int64_t vocab_, hidden_;
+  double base_;
+  Tensor weight_, inv_freq_;
+};
+
 // y = (x * rsqrt(mean(x^2) + eps)) * w in 32-bit (kernels/triton_kernels/rmsnorm.py:63-93); with a residual
 // the norm sees the unrounded sum (kernels/triton_kernels/rmsnorm_residual.py:73-125).
 class RMSNorm : public Norm {
  public:
-  RMSNorm(const PartSpec& s, Kernels& k) : Norm(k), size_(s.integer("size")), eps_((float)s.number("eps")) {}
-  std::vector<ParamDecl> params() const override { return {{"weight", {size_}, true, true, 0.9, 1.1}}; }
+  // offset: the weight that multiplies is offset + w (1 for a weight that is stored around zero, 0 by default).
+  RMSNorm(const PartSpec& s, Kernels& k) : Norm(k), size_(s.integer("size")), eps_((float)s.number("eps")), offset_((float)s.number("offset", 0.0)) {}
+  std::vector<ParamDecl> params() const override {
+    if (offset_ != 0.f) return {{"weight", {size_}, true, true, -0.1, 0.1}};
+    return {{"weight", {size_}, true, true, 0.9, 1.1}};
+  }
   void load(std::map<std::string, Tensor>& t) override { weight_ = need(t, "weight"); }
-  Tensor forward(const Tensor& x) override { return kernels.rmsnorm(x, weight_, eps_); }
-  Tensor forward_add(const Tensor& x, Tensor& residual) override { return kernels.add_rmsnorm(x, residual, weight_, eps_); }
-  const Tensor* row_scale_weight() const override { return &weight_; }
+  // Rows of a 32-bit residual stream are read as they are; the result is elements either way.
+  Tensor forward(const Tensor& x) override {
+    if (offset_ != 0.f || x.dtype != kernels.dtype()) return kernels.stream_norm(x, weight_, eps_, offset_);
+    return kernels.rmsnorm(x, weight_, eps_);
+  }
+  Tensor forward_add(const Tensor& x, Tensor& residual) override {
+    if (offset_ != 0.f) throw EngineError("a norm with a weight offset has no fused residual add in the element type");
+    return kernels.add_rmsnorm(x, residual, weight_, eps_);
+  }
+  void forward_scaled_add(const Tensor& y, const Tensor& base, Tensor& out, float mult) override {
+    kernels.stream_norm_add(out, base, y, weight_, eps_, offset_, mult);
+  }
+  const Tensor* row_scale_weight() const override { return offset_ == 0.f ? &weight_ : nullptr; }
   float eps() const override { return eps_; }
 
  private:
   int64_t size_;
-  float eps_;
+  float eps_, offset_;
   Tensor weight_;
 };
 
@@ -224,21 +323,53 @@ struct AttentionItems {
 // projection.  window > 0 limits a query to that many last keys.  q_norm, k_norm and position are parts of
 // their own; when they are weighted row scales and a rotation by tables the three steps between the projections
 // run as one launch.
+//
+// Further parameters, all optional: value_dim (the values' head size, where it differs from the keys'), bias (q, k
+// and v projections with biases), softcap (score <- softcap * tanh(score / softcap)), keep_first (with a window: the
+// first keys of a sequence stay visible), sink (a learned number per head whose exponential joins the softmax's
+// denominator), exact_weights (the probabilities meet the values in 32-bit), own_kv 0 (the layer has no key and
+// value projections: it always reads another execution's cache).  The cache and the kernels see one head size: the
+// larger of the two, rounded up to 16; the shorter of keys and values is padded with zeros in the weights, so that
+// the projections write the padding and the output projection ignores it.
 class Attention : public Mixer {
  public:
   Attention(const PartSpec& s, Kernels& k)
       : Mixer(k), hidden_(s.integer("hidden_size")), nq_((int)s.integer("num_heads")), nkv_((int)s.integer("num_kv_heads")),
-        d_((int)s.integer("head_dim")), scale_((float)s.number("scale")), window_((int)s.integer("window", 0)) {
+        dk_((int)s.integer("head_dim")), dv_((int)s.integer("value_dim", s.integer("head_dim"))), scale_((float)s.number("scale")),
+        window_((int)s.integer("window", 0)), keep_((int)s.integer("keep_first", 0)), softcap_((float)s.number("softcap", 0.0)),
+        bias_(s.integer("bias", 0) != 0), sink_(s.integer("sink", 0) != 0), exact_(s.integer("exact_weights", 0) != 0),
+        own_kv_(s.integer("own_kv", 1) != 0) {
+    d_ = (int)round_up(std::max(dk_, dv_), 16);
     if (nq_ % nkv_) throw ConfigError(std::to_string(nq_) + " heads are not a multiple of " + std::to_string(nkv_) + " kv heads");
-    if (d_ % 16 || d_ < 16 || d_ > 256)
-      throw ConfigError("head size " + std::to_string(d_) + ": the attention kernels take multiples of 16 from 16 to 256");
+    if (dk_ < 1 || dv_ < 1 || d_ > 256)
+      throw ConfigError("head sizes " + std::to_string(dk_) + " and " + std::to_string(dv_) + ": the attention kernels take up to 256");
+    if (window_ == 0) keep_ = 0;
     if (const PartSpec* p = s.part("q_norm")) q_norm_ = build_part<Norm>("norm", *p, k);
     if (const PartSpec* p = s.part("k_norm")) k_norm_ = build_part<Norm>("norm", *p, k);
     if (const PartSpec* p = s.part("position")) position_ = build_part<PositionEncoding>("position", *p, k);
+    if ((bias_ || d_ != dk_) && (q_norm_ || k_norm_ || position_))
+      throw ConfigError("attention: biases and padded head sizes are not built together with head norms or a position encoding");
   }
+  // The kernel with capped scores serves every one of these.
+  bool capped() const { return softcap_ > 0.f || keep_ > 0 || sink_ || exact_; }
   std::vector<ParamDecl> params() const override {
-    return {{"q_proj.weight", {(int64_t)nq_ * d_, hidden_}}, {"k_proj.weight", {(int64_t)nkv_ * d_, hidden_}},
-            {"v_proj.weight", {(int64_t)nkv_ * d_, hidden_}}, {"o_proj.weight", {hidden_, (int64_t)nq_ * d_}}};
+    std::vector<ParamDecl> p = {{"q_proj.weight", {(int64_t)nq_ * dk_, hidden_}}, {"o_proj.weight", {hidden_, (int64_t)nq_ * dv_}}};
+    if (own_kv_) {
+      p.push_back({"k_proj.weight", {(int64_t)nkv_ * dk_, hidden_}});
+      p.push_back({"v_proj.weight", {(int64_t)nkv_ * dv_, hidden_}});
+    }
+    if (bias_) {
+      p.push_back({"q_proj.bias", {(int64_t)nq_ * dk_}});
+      if (own_kv_) {
+        p.push_back({"k_proj.bias", {(int64_t)nkv_ * dk_}});
+        p.push_back({"v_proj.bias", {(int64_t)nkv_ * dv_}});
+      }
+    }
+    if (sink_) {
+      ParamDecl sinks{"sinks", {(int64_t)nq_}, true, true, -1.0, 1.0};
+      p.push_back(sinks);
+    }
+    return p;
   }
   std::vector<std::pair<std::string, Part*>> children() override {
     std::vector<std::pair<std::string, Part*>> c;
@@ -250,8 +381,24 @@ class Attention : public Mixer {
   void load(std::map<std::string, Tensor>& t) override {
     // One launch projects q, k and v (kernels/triton_kernels/qkv_matmul.py:108-211); rows of the fused
     // weight are q's, then k's, then v's.
-    w_qkv_ = stack_rows({need(t, "q_proj.weight"), need(t, "k_proj.weight"), need(t, "v_proj.weight")});
-    w_o_ = need(t, "o_proj.weight");
+    std::vector<Tensor> rows = {pad_row_blocks(need(t, "q_proj.weight"), nq_, dk_, d_)};
+    if (own_kv_) {
+      rows.push_back(pad_row_blocks(need(t, "k_proj.weight"), nkv_, dk_, d_));
+      rows.push_back(pad_row_blocks(need(t, "v_proj.weight"), nkv_, dv_, d_));
+    }
+    w_qkv_ = rows.size() > 1 ? stack_rows(rows) : rows[0];
+    w_o_ = pad_column_blocks(need(t, "o_proj.weight"), nq_, dv_, d_);
+    if (bias_) {
+      std::vector<Tensor> b = {pad_row_blocks(need(t, "q_proj.bias"), nq_, dk_, d_)};
+      if (own_kv_) {
+        b.push_back(pad_row_blocks(need(t, "k_proj.bias"), nkv_, dk_, d_));
+        b.push_back(pad_row_blocks(need(t, "v_proj.bias"), nkv_, dv_, d_));
+      }
+      for (Tensor& piece : b) piece = piece.view({piece.numel(), 1});
+      b_qkv_ = b.size() > 1 ? stack_rows(b) : b[0];
+      b_qkv_ = b_qkv_.view({b_qkv_.numel()});
+    }
+    if (sink_) sinks_ = need(t, "sinks");
   }
   // Head norms, rotation and cache store run as one launch when the norms are weighted row scales with one eps
   // and the position encoding is a rotation by tables; any other kind runs through its own methods, step by step.
@@ -268,6 +415,7 @@ class Attention : public Mixer {
     n.num_kv_heads = nkv_;
     n.head_dim = d_;
     n.window = window_;
+    n.keep_first = keep_;
     return n;
   }
   const char* step_inputs_key() const override { return "attention.items"; }
@@ -329,9 +477,13 @@ class Attention : public Mixer {
     Tensor ws_t;
     if (gf) ws_t = ctx.workspace(gf);
     const Tensor* ws = gf ? &ws_t : nullptr;
+    if (cache.writable && !own_kv_) throw EngineError("an attention layer without key and value projections was given a cache to write");
     const Tensor qkv = k.gemm(x, cache.writable ? w_qkv_ : w_qkv_.rows(0, (int64_t)nq_ * d_), ws);
     Tensor q;
-    if (fused()) {
+    if (bias_) {
+      const int64_t bw = (int64_t)(nq_ + (cache.writable ? 2 * nkv_ : 0)) * d_;
+      q = k.qkv_post_bias(qkv, nq_, cache.writable ? nkv_ : 0, d_, &cache.k, &cache.v, cache.page_size, &tables.slots, b_qkv_.rows(0, bw));
+    } else if (fused()) {
       const Norm* en = q_norm_ ? q_norm_.get() : k_norm_.get();
       q = k.qkv_post(qkv, nq_, cache.writable ? nkv_ : 0, d_, &cache.k, &cache.v, cache.page_size,
                      q_norm_ ? q_norm_->row_scale_weight() : nullptr, k_norm_ ? k_norm_->row_scale_weight() : nullptr,
@@ -344,13 +496,23 @@ class Attention : public Mixer {
     AttentionItems& m = items(*ctx.host);
     const Tensor& prefill_items = ctx.inputs.at("attention.prefill_items");
     const Tensor& decode_items = ctx.inputs.at("attention.decode_items");
-    if (prefill_items.dim(0))
-      k.paged_attention(out, q, cache.k, cache.v, tables.block_table, ctx.cu_q, ctx.k_len, prefill_items, 0, scale_, window_,
-                        ctx.host->k_len_bound, 0, nullptr);
+    const Tensor* sinks = sink_ ? &sinks_ : nullptr;
+    if (prefill_items.dim(0)) {
+      if (capped())
+        k.paged_attention_capped(out, q, cache.k, cache.v, tables.block_table, ctx.cu_q, ctx.k_len, prefill_items, 0, scale_, window_, keep_,
+                                 softcap_, sinks, ctx.host->k_len_bound, 0, nullptr);
+      else
+        k.paged_attention(out, q, cache.k, cache.v, tables.block_table, ctx.cu_q, ctx.k_len, prefill_items, 0, scale_, window_,
+                          ctx.host->k_len_bound, 0, nullptr);
+    }
     if (decode_items.dim(0)) {
       const Tensor scratch = ctx.workspace(k.attn_scratch_floats((int)decode_items.dim(0), nq_, d_, m.nseg));
-      k.paged_attention(out, q, cache.k, cache.v, tables.block_table, ctx.cu_q, ctx.k_len, decode_items, 1, scale_, window_,
-                        m.decode_bound, m.nseg, &scratch);
+      if (capped())
+        k.paged_attention_capped(out, q, cache.k, cache.v, tables.block_table, ctx.cu_q, ctx.k_len, decode_items, 1, scale_, window_, keep_,
+                                 softcap_, sinks, m.decode_bound, m.nseg, &scratch);
+      else
+        k.paged_attention(out, q, cache.k, cache.v, tables.block_table, ctx.cu_q, ctx.k_len, decode_items, 1, scale_, window_,
+                          m.decode_bound, m.nseg, &scratch);
     }
     return k.gemm(out.view({T, (int64_t)nq_ * d_}), w_o_, ws);
   }
@@ -377,12 +539,14 @@ class Attention : public Mixer {
   }
 
   int64_t hidden_;
-  int nq_, nkv_, d_;
+  int nq_, nkv_, dk_, dv_, d_ = 0;   // d_: the head size of the cache and the kernels
   float scale_;
-  int window_;
+  int window_, keep_;
+  float softcap_;
+  bool bias_, sink_, exact_, own_kv_;
   std::unique_ptr<Norm> q_norm_, k_norm_;
   std::unique_ptr<PositionEncoding> position_;
-  Tensor w_qkv_, w_o_;
+  Tensor w_qkv_, w_o_, b_qkv_, sinks_;
 };
 
 // down(silu(gate(x)) * up(x)) without biases (src/exec/dense_swiglu_decoder.rs:396-438); gate and up are one
@@ -457,14 +621,207 @@ class PreNormBlock : public Block {
 // parts the one tensor (python/vosti_kernels/model_families/qwen3/physical.py:131-134).
 class LinearHead : public Head {
  public:
-  LinearHead(const PartSpec& s, Kernels& k) : Head(k), vocab_(s.integer("vocab_size")), hidden_(s.integer("hidden_size")) {}
+  // softcap > 0: logits <- softcap * tanh(logits / softcap).
+  LinearHead(const PartSpec& s, Kernels& k)
+      : Head(k), vocab_(s.integer("vocab_size")), hidden_(s.integer("hidden_size")), softcap_((float)s.number("softcap", 0.0)) {}
   std::vector<ParamDecl> params() const override { return {{"weight", {vocab_, hidden_}}}; }
   void load(std::map<std::string, Tensor>& t) override { weight_ = need(t, "weight"); }
-  Tensor forward(const Tensor& x) override { return kernels.gemm(x, weight_); }
+  Tensor forward(const Tensor& x) override {
+    Tensor logits = kernels.gemm(x, weight_);
+    if (softcap_ > 0.f) kernels.softcap(logits, softcap_);
+    return logits;
+  }
 
  private:
   int64_t vocab_, hidden_;
+  float softcap_;
   Tensor weight_;
+};
+
+// The gated delta rule with one decay per head and key channel.  For the mixer's input h:
+//   q = W_q h, k = W_k h (kv heads x key size), v = W_v h (heads x value size), each through a short causal
+//   convolution per channel (taps [channels, K], the last tap the current token's, zeros before a sequence's start)
+//   and silu; q and k become unit vectors per head (x / sqrt(sum(x^2) + unit_eps)), q times key size^(-1/2);
+//   beta = sigmoid(W_b h) per head; g = exp(-exp(A_log[head]) * softplus(W_a2 (W_a1 h) + dt_bias)) per head and key
+//   channel; per head, token by token:  S <- diag(g) S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q;
+//   y = o / sqrt(mean(o^2) + eps) * w_norm * sigmoid(W_g2 (W_g1 h)) per head; out = W_o y.
+// A request's state slot holds the heads' S in 32-bit and the last K - 1 inputs of the three convolutions.  The six
+// input projections are one launch (their weights stacked, each section padded to a multiple of 8 rows with zero
+// rows, so that the low-rank pairs' second halves read their columns in place); conv, norms, decays, recurrence and
+// read-out are kernels of delta.hip, all in 32-bit.
+class ChannelDelta : public Mixer {
+ public:
+  ChannelDelta(const PartSpec& s, Kernels& k)
+      : Mixer(k), hidden_(s.integer("hidden_size")), H_((int)s.integer("num_heads")), G_((int)s.integer("num_kv_heads")),
+        d_((int)s.integer("key_dim")), dv_((int)s.integer("value_dim")), taps_((int)s.integer("conv_taps")),
+        decay_rank_(s.integer("decay_rank", 0)), gate_rank_(s.integer("gate_rank", 0)), eps_((float)s.number("eps")),
+        unit_eps_((float)s.number("unit_eps", 1e-6)) {
+    if (H_ % G_) throw ConfigError(std::to_string(H_) + " heads are not a multiple of " + std::to_string(G_) + " kv heads");
+    if (taps_ < 1 || taps_ > 17) throw ConfigError("a short convolution of " + std::to_string(taps_) + " taps: 1 to 17 are built");
+    qk_ = round_up((int64_t)G_ * d_, 8);
+    v_ = round_up((int64_t)H_ * dv_, 8);
+    channels_ = 2 * qk_ + v_;
+  }
+  std::vector<ParamDecl> params() const override {
+    const int64_t qk = (int64_t)G_ * d_, v = (int64_t)H_ * dv_, hd = (int64_t)H_ * d_;
+    // 0: the rank is whatever the stored tensors have.
+    const int64_t ra = decay_rank_ > 0 ? decay_rank_ : -1, rg = gate_rank_ > 0 ? gate_rank_ : -1;
+    auto uniform = [](const char* name, std::vector<int64_t> shape, double lo, double hi) {
+      ParamDecl p{name, std::move(shape), true, true, lo, hi};
+      return p;
+    };
+    ParamDecl taps_q{"q_conv.weight", {qk, taps_}}, taps_k{"k_conv.weight", {qk, taps_}}, taps_v{"v_conv.weight", {v, taps_}};
+    taps_q.p0 = taps_k.p0 = taps_v.p0 = 0.3;
+    ParamDecl q{"q_proj.weight", {qk, hidden_}}, kk{"k_proj.weight", {qk, hidden_}}, vv{"v_proj.weight", {v, hidden_}};
+    q.p0 = kk.p0 = vv.p0 = 0.1;
+    ParamDecl a1{"decay_down.weight", {ra, hidden_}}, a2{"decay_up.weight", {hd, ra}}, g1{"gate_down.weight", {rg, hidden_}}, g2{"gate_up.weight", {v, rg}};
+    a1.free_size = a2.free_size = g1.free_size = g2.free_size = std::max<int64_t>(8, hidden_ / 16);
+    return {q, taps_q, kk, taps_k, vv, taps_v, {"beta_proj.weight", {(int64_t)H_, hidden_}}, uniform("A_log", {(int64_t)H_}, -1.0, 1.0),
+            uniform("out_norm.weight", {(int64_t)dv_}, 0.9, 1.1), a1, a2, uniform("dt_bias", {hd}, -1.0, 1.0), g1, g2,
+            {"o_proj.weight", {hidden_, v}}};
+  }
+  void load(std::map<std::string, Tensor>& t) override {
+    const Tensor a1 = need(t, "decay_down.weight"), a2 = need(t, "decay_up.weight"), g1 = need(t, "gate_down.weight"), g2 = need(t, "gate_up.weight");
+    if (a1.dim(0) != a2.dim(1) || g1.dim(0) != g2.dim(1))
+      throw EngineError("the delta rule's low-rank projections do not fit each other: " + a1.describe() + " with " + a2.describe() + ", " +
+                        g1.describe() + " with " + g2.describe());
+    const int64_t ra = round_up(a1.dim(0), 8), rg = round_up(g1.dim(0), 8), nb = round_up(H_, 8);
+    const int64_t qk = (int64_t)G_ * d_, v = (int64_t)H_ * dv_;
+    w_in_ = stack_rows({pad_matrix(need(t, "q_proj.weight"), qk_, hidden_), pad_matrix(need(t, "k_proj.weight"), qk_, hidden_),
+                        pad_matrix(need(t, "v_proj.weight"), v_, hidden_), pad_matrix(need(t, "beta_proj.weight"), nb, hidden_),
+                        pad_matrix(a1, ra, hidden_), pad_matrix(g1, rg, hidden_)});
+    beta_col_ = channels_;
+    decay_col_ = beta_col_ + nb;
+    gate_col_ = decay_col_ + ra;
+    w_decay_up_ = pad_matrix(a2, a2.dim(0), ra);
+    w_gate_up_ = pad_matrix(g2, g2.dim(0), rg);
+    conv_ = stack_rows({pad_matrix(need(t, "q_conv.weight"), qk_, taps_), pad_matrix(need(t, "k_conv.weight"), qk_, taps_),
+                        pad_matrix(need(t, "v_conv.weight"), v_, taps_)});
+    (void)qk; (void)v;
+    A_log_ = need(t, "A_log");
+    dt_bias_ = need(t, "dt_bias");
+    out_norm_ = need(t, "out_norm.weight");
+    w_o_ = need(t, "o_proj.weight");
+  }
+  CacheNeed cache_need() const override {
+    CacheNeed n;
+    n.kind = CacheNeed::State;
+    n.state_shape = {state_floats() + (int64_t)(taps_ - 1) * channels_};
+    n.state_dtype = DType::F32;
+    return n;
+  }
+  // Which sequence of the step every token belongs to.
+  const char* step_inputs_key() const override { return "delta.token_seq"; }
+  void step_inputs(HostStep& step, std::vector<std::pair<std::string, HostArray>>& out) override {
+    HostArray a;
+    for (size_t s = 0; s < step.q_lens.size(); ++s) a.data.insert(a.data.end(), (size_t)step.q_lens[s], (int32_t)s);
+    a.shape = {(int64_t)a.data.size()};
+    out.emplace_back("delta.token_seq", std::move(a));
+  }
+
+  Tensor forward(const Tensor& x, StepContext& ctx, CacheEntry& cache) override {
+    if (cache.kind != CacheNeed::State) throw EngineError("the delta rule was handed a cache entry without state");
+    Kernels& k = kernels;
+    const Tensor proj = k.gemm(x, w_in_);
+    const Tensor a = k.gemm_columns(proj, decay_col_, w_decay_up_);
+    const Tensor gate = k.gemm_columns(proj, gate_col_, w_gate_up_);
+    Tensor qkv = k.delta_conv(proj, conv_, cache.state, state_floats(), ctx.inputs.at("delta.token_seq"), ctx.cu_q, ctx.positions, ctx.state_slots);
+    k.delta_unit(qkv, 0, G_, d_, unit_eps_, 1.f / std::sqrt((float)d_));
+    k.delta_unit(qkv, qk_, G_, d_, unit_eps_, 1.f);
+    const Tensor decay = k.delta_decay(a, dt_bias_, A_log_, H_, d_);
+    const Tensor o = k.delta_rule(qkv, 0, (int)qk_, (int)(2 * qk_), decay, proj, beta_col_, cache.state, ctx.cu_q, ctx.positions, ctx.state_slots,
+                                  H_, G_, d_, dv_);
+    return k.gemm(k.delta_out(o, gate, out_norm_, H_, dv_, eps_), w_o_);
+  }
+
+ private:
+  int64_t state_floats() const { return (int64_t)H_ * d_ * dv_; }
+  int64_t hidden_;
+  int H_, G_, d_, dv_, taps_;
+  int64_t decay_rank_, gate_rank_;
+  float eps_, unit_eps_;
+  int64_t qk_ = 0, v_ = 0, channels_ = 0, beta_col_ = 0, decay_col_ = 0, gate_col_ = 0;
+  Tensor w_in_, w_decay_up_, w_gate_up_, conv_, A_log_, dt_bias_, out_norm_, w_o_;
+};
+
+// A layer without a feed-forward names this kind; an arrangement that allows it never calls it.
+class NoFeedForward : public FeedForward {
+ public:
+  NoFeedForward(const PartSpec&, Kernels& k) : FeedForward(k) {}
+  Tensor forward(const Tensor&, StepContext&) override { throw EngineError("a layer without a feed-forward was asked to run one"); }
+};
+
+// A residual stream x in 32-bit, a norm before and after each sublayer, and a weighted sum over the stream's earlier
+// states at the layer's end:
+//   x <- x + m * norm_mixer_out(mixer(norm_mixer_in(x)));  x <- x + m * norm_ffn_out(ffn(norm_ffn_in(x))) (if the
+//   layer has a feed-forward);  X_(i+1) = x;  passed on: sum over j <= i + 1 of depth_weights[j] * X_j,
+// where X_0 is what the embedding gave and i = `depth`, the layer's place in the run order.  The states of a step lie
+// in one tensor [states, tokens, width] that the first layer of the step takes from the arena (ctx.carry).
+class SandwichDepthBlock : public Block {
+ public:
+  SandwichDepthBlock(Kernels& k, std::unique_ptr<Mixer> mixer, std::unique_ptr<FeedForward> ffn, std::map<std::string, std::unique_ptr<Norm>> norms,
+                     const std::map<std::string, double>& numbers)
+      : Block(k), mixer_(std::move(mixer)), ffn_(std::move(ffn)), norms_(std::move(norms)) {
+    auto number = [&](const char* name) {
+      auto it = numbers.find(name);
+      if (it == numbers.end()) throw ConfigError(std::string("a sandwich_depth block needs the number '") + name + "'");
+      return it->second;
+    };
+    mult_ = (float)number("residual_mult");
+    depth_ = (int)number("depth");
+    states_ = (int)number("states");
+    hidden_ = (int64_t)number("hidden_size");
+    if (depth_ < 0 || depth_ + 1 >= states_) throw ConfigError("a sandwich_depth block at depth " + std::to_string(depth_) + " of " + std::to_string(states_) + " states");
+    has_ffn_ = dynamic_cast<NoFeedForward*>(ffn_.get()) == nullptr;
+    for (const char* n : {"mixer_in", "mixer_out"})
+      if (!norms_.count(n)) throw ConfigError(std::string("a sandwich_depth block needs the norms 'mixer_in' and 'mixer_out'; missing: ") + n);
+    if (has_ffn_ && (!norms_.count("ffn_in") || !norms_.count("ffn_out")))
+      throw ConfigError("a sandwich_depth block with a feed-forward needs the norms 'ffn_in' and 'ffn_out'");
+  }
+  std::vector<ParamDecl> params() const override {
+    ParamDecl w{"depth_weights", {(int64_t)depth_ + 2}, true, true, 0.0, 2.0 / (depth_ + 2)};
+    return {w};
+  }
+  void load(std::map<std::string, Tensor>& t) override { weights_ = need(t, "depth_weights"); }
+  std::vector<std::pair<std::string, Part*>> children() override {
+    std::vector<std::pair<std::string, Part*>> c = {{"mixer", mixer_.get()}, {"feed_forward", ffn_.get()}};
+    for (auto& n : norms_) c.emplace_back("norms." + n.first, n.second.get());
+    return c;
+  }
+  Mixer& mixer() override { return *mixer_; }
+  std::pair<Tensor, Tensor> forward(const Tensor& hidden, Tensor residual, StepContext& ctx, CacheEntry& cache) override {
+    Kernels& k = kernels;
+    if (hidden.dtype != DType::F32 || hidden.shape.size() != 2 || hidden.dim(1) != hidden_)
+      throw EngineError("a sandwich_depth block takes the 32-bit residual stream, not " + hidden.describe());
+    const int64_t T = hidden.dim(0);
+    Tensor& states = ctx.carry["stream.states"];
+    if (depth_ == 0) {
+      states = k.empty({(int64_t)states_, T, hidden_}, DType::F32);
+      hip_check(hipMemcpyAsync(states.data, hidden.data, hidden.bytes(), hipMemcpyDeviceToDevice, k.stream), "keeping the embedding's output");
+    }
+    if (!states.data || states.dim(0) != states_ || states.dim(1) != T) throw EngineError("a sandwich_depth block found no states of this step's stream");
+    Tensor result = states.rows(depth_ + 1, 1).view({T, hidden_});
+    const Tensor mixed = mixer_->forward(norms_["mixer_in"]->forward(hidden), ctx, cache);
+    if (has_ffn_) {
+      Tensor mid = k.empty({T, hidden_}, DType::F32);
+      norms_["mixer_out"]->forward_scaled_add(mixed, hidden, mid, mult_);
+      const Tensor fed = ffn_->forward(norms_["ffn_in"]->forward(mid), ctx);
+      norms_["ffn_out"]->forward_scaled_add(fed, mid, result, mult_);
+    } else {
+      norms_["mixer_out"]->forward_scaled_add(mixed, hidden, result, mult_);
+    }
+    return {k.stream_mix(states, weights_, depth_ + 2), residual};
+  }
+
+ private:
+  std::unique_ptr<Mixer> mixer_;
+  std::unique_ptr<FeedForward> ffn_;
+  std::map<std::string, std::unique_ptr<Norm>> norms_;
+  float mult_ = 1.f;
+  int depth_ = 0, states_ = 0;
+  int64_t hidden_ = 0;
+  bool has_ffn_ = true;
+  Tensor weights_;
 };
 
 template <class T>
@@ -478,13 +835,20 @@ void register_standard_parts() {
   static std::once_flag once;
   std::call_once(once, [] {
     register_part("embedding", "token_embedding", factory<TokenEmbedding>());
+    register_part("embedding", "token_embedding_sinusoid", factory<SinusoidEmbedding>());
+    register_part("mixer", "channel_delta", factory<ChannelDelta>());
+    register_part("feed_forward", "none", factory<NoFeedForward>());
+    register_block("sandwich_depth", [](Kernels& k, std::unique_ptr<Mixer> m, std::unique_ptr<FeedForward> f,
+                                        std::map<std::string, std::unique_ptr<Norm>> n, const std::map<std::string, double>& numbers) {
+      return std::unique_ptr<Block>(new SandwichDepthBlock(k, std::move(m), std::move(f), std::move(n), numbers));
+    });
     register_part("norm", "rmsnorm", factory<RMSNorm>());
     register_part("position", "rotary", factory<Rotary>());
     register_part("mixer", "attention", factory<Attention>());
     register_part("feed_forward", "swiglu", factory<SwiGLU>());
     register_part("head", "linear_head", factory<LinearHead>());
     register_block("prenorm", [](Kernels& k, std::unique_ptr<Mixer> m, std::unique_ptr<FeedForward> f,
-                                 std::map<std::string, std::unique_ptr<Norm>> n) {
+                                 std::map<std::string, std::unique_ptr<Norm>> n, const std::map<std::string, double>&) {
       return std::unique_ptr<Block>(new PreNormBlock(k, std::move(m), std::move(f), std::move(n)));
     });
   });

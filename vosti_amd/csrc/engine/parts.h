@@ -20,11 +20,12 @@ namespace vosti {
 
 struct ParamDecl {
   std::string name;               // local name, e.g. "q_proj.weight"
-  std::vector<int64_t> shape;
+  std::vector<int64_t> shape;     // -1: a size that the stored tensor gives (the part checks it when it loads)
   bool keep_f32 = false;          // a tensor the file stores in 32-bit stays so
   // Random weights: approximately normal with this standard deviation, or (uniform) in [lo, hi).
   bool uniform = false;
   double p0 = 0.02, p1 = 0.0;     // normal: p0 = standard deviation; uniform: p0 = lo, p1 = hi
+  int64_t free_size = 8;          // what a size of -1 becomes when the weights are drawn and no file gives it
 };
 
 struct HostArray {
@@ -53,6 +54,7 @@ struct StepContext {
   std::vector<GroupTables> groups;
   HostStep* host = nullptr;
   std::map<std::string, Tensor> inputs;              // the arrays parts asked for, on the GPU
+  std::map<std::string, Tensor> carry;               // what a part leaves for later parts of the same step (empty at its start)
   std::function<Tensor(int64_t)> workspace;           // float32 scratch of at least that many elements
 };
 
@@ -60,6 +62,7 @@ struct StepContext {
 struct CacheNeed {
   enum Kind { None, Pages, State } kind = None;
   int num_kv_heads = 0, head_dim = 0, window = 0;    // Pages
+  int keep_first = 0;                                // Pages with a window: the first keys that stay visible and are never given back
   std::vector<int64_t> state_shape;                  // State: per request
   DType state_dtype = DType::F32;
 };
@@ -96,6 +99,8 @@ class Embedding : public Part {
  public:
   using Part::Part;
   virtual Tensor forward(const Tensor& ids) = 0;
+  // An embedding that needs the step's numbers (positions, say) overrides this one; the model calls it.
+  virtual Tensor forward(const Tensor& ids, StepContext& ctx) { (void)ctx; return forward(ids); }
 };
 
 class Norm : public Part {
@@ -107,6 +112,8 @@ class Norm : public Part {
   // A norm that is y = x * rsqrt(mean(x^2) + eps) * w says so; a mixer may then run it inside a launch of its own.
   virtual const Tensor* row_scale_weight() const { return nullptr; }
   virtual float eps() const { return 0.f; }
+  // out = base + mult * norm(y) on a residual stream that is kept in 32-bit; out may be base.
+  virtual void forward_scaled_add(const Tensor& y, const Tensor& base, Tensor& out, float mult);
 };
 
 class PositionEncoding : public Part {
@@ -148,8 +155,9 @@ class Block : public Part {
 };
 
 using PartFactory = std::function<std::unique_ptr<Part>(const PartSpec&, Kernels&)>;
+// The last argument: the layer's own numbers (LayerSpec::block_numbers), for arrangements that have constants.
 using BlockFactory = std::function<std::unique_ptr<Block>(Kernels&, std::unique_ptr<Mixer>, std::unique_ptr<FeedForward>,
-                                                          std::map<std::string, std::unique_ptr<Norm>>)>;
+                                                          std::map<std::string, std::unique_ptr<Norm>>, const std::map<std::string, double>&)>;
 // category: "embedding", "norm", "position", "mixer", "feed_forward", "head".
 void register_part(const std::string& category, const std::string& kind, PartFactory make);
 void register_block(const std::string& kind, BlockFactory make);
@@ -165,7 +173,7 @@ std::unique_ptr<T> build_part(const std::string& category, const PartSpec& spec,
   return std::unique_ptr<T>(t);
 }
 
-void register_standard_parts();   // the kinds the Qwen3 dense decoder is made of
+void register_standard_parts();   // the kinds the built-in architectures are made of
 bool part_registered(const std::string& category, const std::string& kind);
 bool block_registered(const std::string& kind);
 // Why this registry cannot build the model, or "" if it can: the first part or block kind that is missing.

@@ -21,15 +21,20 @@ static Tensor zeroed(std::vector<int64_t> shape, DType t) {
 CachePool::CachePool(DecoderModel& model, int page_size_, int num_pages, int num_slots, bool prefix_cache) : page_size(page_size_) {
   if (page_size < 8 || (page_size & (page_size - 1))) throw EngineError("page size " + std::to_string(page_size) + " must be a power of two, at least 8");
   const std::vector<CacheNeed> needs = model.cache_needs();
+  std::vector<std::pair<int, int>> kinds;                    // (window, kept first keys)
   for (const CacheNeed& n : needs) {
-    if (n.kind == CacheNeed::Pages && std::find(group_windows.begin(), group_windows.end(), n.window) == group_windows.end())
-      group_windows.push_back(n.window);
+    const std::pair<int, int> kind{n.window, n.window ? n.keep_first : 0};
+    if (n.kind == CacheNeed::Pages && std::find(kinds.begin(), kinds.end(), kind) == kinds.end()) kinds.push_back(kind);
     if (n.kind == CacheNeed::State) has_state = true;
   }
-  std::sort(group_windows.begin(), group_windows.end());     // 0 (all keys) first
-  if (group_windows.empty()) group_windows.push_back(0);
+  std::sort(kinds.begin(), kinds.end());                     // 0 (all keys) first
+  if (kinds.empty()) kinds.push_back({0, 0});
   std::vector<GroupSpec> groups;
-  for (int w : group_windows) groups.push_back({w, num_pages});
+  for (const auto& kind : kinds) {
+    group_windows.push_back(kind.first);
+    group_keeps.push_back(kind.second);
+    groups.push_back({kind.first, num_pages, kind.second});
+  }
   // A prefix page holds keys only; a mixer with state of its own could not resume from it.
   manager_ = std::make_unique<CacheManager>(page_size, groups, num_slots, prefix_cache && !has_state);
   const DType dtype = model.kernels().dtype();
@@ -45,7 +50,7 @@ CachePool::CachePool(DecoderModel& model, int page_size_, int num_pages, int num
       e.writable = false;
     } else if (n.kind == CacheNeed::Pages) {
       e.kind = CacheNeed::Pages;
-      e.group = (int)(std::find(group_windows.begin(), group_windows.end(), n.window) - group_windows.begin());
+      e.group = (int)(std::find(kinds.begin(), kinds.end(), std::pair<int, int>{n.window, n.window ? n.keep_first : 0}) - kinds.begin());
       e.page_size = page_size;
       e.k = zeroed({num_pages, n.num_kv_heads, page_size, n.head_dim}, dtype);
       e.v = zeroed({num_pages, n.num_kv_heads, n.head_dim, page_size}, dtype);

@@ -39,7 +39,8 @@ class CachePool {
   CachePool(DecoderModel& model, int page_size, int num_pages, int num_slots, bool prefix_cache);
   CacheManager& manager() { return *manager_; }
   std::vector<CacheEntry> entries;          // one per schedule entry
-  std::vector<int> group_windows;
+  std::vector<int> group_windows;           // one entry per group; groups differ in (window, kept first keys)
+  std::vector<int> group_keeps;
   int page_size;
   bool has_state = false;
   size_t bytes() const { return bytes_; }

@@ -12,6 +12,7 @@ CacheManager::CacheManager(int page_size, std::vector<GroupSpec> groups, int num
   for (const GroupSpec& s : groups) {
     Group g;
     g.window = s.window;
+    g.keep_first = s.window != 0 ? s.keep_first : 0;
     g.num_pages = s.num_pages;
     for (int p = 0; p < s.num_pages; ++p) g.free.push_back(p);
     g.holders.assign(s.num_pages, PAGE_FREE);
@@ -229,7 +230,9 @@ void CacheManager::release_window(Request& r) {
     // The next query stands at position >= length and sees keys >= length - w + 1.
     const int first_needed = std::max(0, r.length - w + 1);
     const int upto = std::min((int)r.pages[g].size(), first_needed / page_size_);
-    for (int j = r.first_live[g]; j < upto; ++j) {
+    // The pages of the first keys that every later query still sees stay.
+    const int kept = (groups_[g].keep_first + page_size_ - 1) / page_size_;
+    for (int j = std::max(r.first_live[g], kept); j < upto; ++j) {
       if (r.pages[g][j] >= 0) {
         give_page(g, r.pages[g][j]);
         r.pages[g][j] = -1;

@@ -5,7 +5,8 @@
 // the engine.
 //
 // Groups.  Layers with the same need share a group: a group keeps all keys of a
-// request (window == 0) or only the last `window` of them.  Each group has its
+// request (window == 0) or only the last `window` of them, and with those the
+// first `keep_first`.  Each group has its
 // own pool of pages and its own block table per request; all groups use one
 // page size.  Position i of a request lives in logical page i / page_size of
 // each group, at slot  page * page_size + i % page_size.
@@ -53,6 +54,7 @@ enum Status : int {
 struct GroupSpec {
   int window;     // 0: the group keeps every key
   int num_pages;
+  int keep_first = 0;   // with a window: the pages that hold a request's first keep_first keys are never given back
 };
 
 class CacheManager {
@@ -70,6 +72,7 @@ class CacheManager {
   int page_size() const { return page_size_; }
   int num_groups() const { return (int)groups_.size(); }
   int window(int group) const { return groups_[group].window; }
+  int keep_first(int group) const { return groups_[group].keep_first; }
   int length(RequestId id) const;        // tokens committed
   int pending(RequestId id) const;       // tokens of the step in flight
   int state_slot(RequestId id) const;
@@ -105,6 +108,7 @@ class CacheManager {
  private:
   struct Group {
     int window;
+    int keep_first;
     int num_pages;
     std::deque<int> free;
     std::vector<int> holders;   // per page, its state: PAGE_FREE (in the free queue), PAGE_PRIVATE (one request's own) or PAGE_NODE (in a prefix node)

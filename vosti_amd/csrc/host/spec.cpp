@@ -75,15 +75,15 @@ std::string names_json(const std::map<std::string, std::string>& names) {
   return out + "}";
 }
 
+std::string numbers_json(const std::map<std::string, double>& numbers) {
+  std::string out = "{";
+  for (const auto& n : numbers) out += (out.size() > 1 ? ", " : "") + json_string(n.first) + ": " + json_number(n.second);
+  return out + "}";
+}
+
 std::string part_json(const PartSpec& p) {
-  std::string out = "{\"kind\": " + json_string(p.kind) + ", \"numbers\": {";
+  std::string out = "{\"kind\": " + json_string(p.kind) + ", \"numbers\": " + numbers_json(p.numbers) + ", \"parts\": {";
   bool first = true;
-  for (const auto& n : p.numbers) {
-    out += (first ? "" : ", ") + json_string(n.first) + ": " + json_number(n.second);
-    first = false;
-  }
-  out += "}, \"parts\": {";
-  first = true;
   for (const auto& c : p.parts) {
     out += (first ? "" : ", ") + json_string(c.first) + ": " + part_json(*c.second);
     first = false;
@@ -104,7 +104,7 @@ std::string model_spec_json(const ModelSpec& spec) {
     out += i ? ", {" : "{";
     size_t same = i;
     for (size_t j = 0; j < i; ++j)
-      if (spec.layers[j].block == l.block && spec.layers[j].mixer == l.mixer && spec.layers[j].feed_forward == l.feed_forward &&
+      if (spec.layers[j].block == l.block && spec.layers[j].block_numbers == l.block_numbers && spec.layers[j].mixer == l.mixer && spec.layers[j].feed_forward == l.feed_forward &&
           spec.layers[j].norms == l.norms) {
         same = j;
         break;
@@ -112,7 +112,7 @@ std::string model_spec_json(const ModelSpec& spec) {
     if (same != i) {
       out += "\"same_as\": " + std::to_string(same);
     } else {
-      out += "\"block\": " + json_string(l.block) + ", \"mixer\": " + part_json(*l.mixer) + ", \"feed_forward\": " + part_json(*l.feed_forward) +
+      out += "\"block\": " + json_string(l.block) + ", \"block_numbers\": " + numbers_json(l.block_numbers) + ", \"mixer\": " + part_json(*l.mixer) + ", \"feed_forward\": " + part_json(*l.feed_forward) +
              ", \"norms\": {";
       bool first = true;
       for (const auto& n : l.norms) {
@@ -157,6 +157,8 @@ std::map<std::string, std::string> model_types() {
 static std::string architecture_name(const Json& config) {
   const Json* archs = config.get("architectures");
   const Json* mt = config.get("model_type");
+  const Json* one = config.get("architecture");
+  if (one && one->kind == Json::String && registry().count(one->text)) return one->text;
   if (archs && archs->kind == Json::Array && !archs->items.empty() && archs->items[0].kind == Json::String) return archs->items[0].text;
   if (mt && mt->kind == Json::String && model_types().count(mt->text)) return model_types()[mt->text];
   return "";

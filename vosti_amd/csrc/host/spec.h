@@ -34,6 +34,7 @@ using PartSpecPtr = std::shared_ptr<const PartSpec>;
 // path inside the layer ("mixer.q_proj.weight", "norms.input.weight") to the tensor's name in the files.
 struct LayerSpec {
   std::string block;
+  std::map<std::string, double> block_numbers;       // constants of the arrangement itself, if it has any
   PartSpecPtr mixer, feed_forward;
   std::map<std::string, PartSpecPtr> norms;
   std::map<std::string, std::string> names;

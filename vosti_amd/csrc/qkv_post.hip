@@ -23,6 +23,7 @@ struct QkvPostArgs {
   elem_t* vc;             // [pages, nkv, d, P]
   const void* q_w;        // [d] or null
   const void* k_w;        // [d] or null
+  const elem_t* bias;     // [(nq + 2 nkv) d] or null: added to the row first (the sum rounded to the element type)
   const elem_t* cos_t;    // [max_pos, rot_half] or null
   const elem_t* sin_t;
   const int32_t* positions;  // [T]
@@ -58,6 +59,7 @@ __global__ __launch_bounds__(256) void qkv_post_kernel(QkvPostArgs a, int per_wa
     for (int i = 0; i < 4; ++i) {
       const int c = lane + 64 * i;
       xv[i] = c < d ? to_f32(x[c]) : 0.f;
+      if (a.bias != nullptr && live && c < d) xv[i] = round_to_elem(xv[i] + to_f32(a.bias[(int64_t)hh * d + c]));
       part = part + xv[i] * xv[i];
     }
     if (w != nullptr) {
@@ -153,6 +155,12 @@ __global__ __launch_bounds__(256) void qkv_post_vec_kernel(QkvPostArgs a, int pe
     const void* w = kind == 0 ? a.q_w : (kind == 1 ? a.k_w : nullptr);
     float xv[VK_VEC];
     load_elems(x, xv);
+    if (a.bias != nullptr && live) {
+      float bv[VK_VEC];
+      load_elems(a.bias + (int64_t)hh * d + j * VK_VEC, bv);
+#pragma unroll
+      for (int e = 0; e < VK_VEC; ++e) xv[e] = round_to_elem(xv[e] + bv[e]);
+    }
     if (w != nullptr) {
       float part = 0.f;
 #pragma unroll
@@ -210,10 +218,10 @@ extern "C" {
 // only q rows (a plain norm and/or rotation of [T, nq, d]).  nq == 0: only the
 // store.  Positions must lie below the tables' row count and slots inside the
 // cache; the caller checks both on the host before the upload.
-int vk_qkv_post(const elem_t* qkv, int64_t row_stride, elem_t* q_out, elem_t* kc, elem_t* vc, const void* q_w,
-                const void* k_w, int w_is_f32, const elem_t* cos_t, const elem_t* sin_t, int rot_half,
-                const int32_t* positions, const int32_t* slots, int T, int nq, int nkv, int d, int P, float eps,
-                hipStream_t st) {
+static int qkv_post_launch(const elem_t* qkv, int64_t row_stride, elem_t* q_out, elem_t* kc, elem_t* vc, const void* q_w,
+                           const void* k_w, int w_is_f32, const elem_t* cos_t, const elem_t* sin_t, int rot_half,
+                           const int32_t* positions, const int32_t* slots, int T, int nq, int nkv, int d, int P, float eps,
+                           const elem_t* bias, hipStream_t st) {
   VK_REQUIRE(T >= 0 && nq >= 0 && nkv >= 0 && nq + nkv > 0, "qkv_post: bad sizes T=%d nq=%d nkv=%d", T, nq, nkv);
   VK_REQUIRE(d > 0 && d <= 256, "qkv_post: head size %d must be in 1..256", d);
   VK_REQUIRE(row_stride >= (int64_t)(nq + 2 * nkv) * d, "qkv_post: row stride %lld too small", (long long)row_stride);
@@ -225,14 +233,14 @@ int vk_qkv_post(const elem_t* qkv, int64_t row_stride, elem_t* q_out, elem_t* kc
   if (T == 0) return 0;
   QkvPostArgs a;
   a.qkv = qkv; a.row_stride = row_stride; a.q_out = q_out; a.kc = kc; a.vc = vc; a.q_w = q_w; a.k_w = k_w;
-  a.cos_t = cos_t; a.sin_t = sin_t; a.positions = positions; a.slots = slots; a.w_is_f32 = w_is_f32;
+  a.cos_t = cos_t; a.sin_t = sin_t; a.positions = positions; a.slots = slots; a.w_is_f32 = w_is_f32; a.bias = bias;
   a.nq = nq; a.nkv = nkv; a.d = d; a.P = P; a.rot_half = rot_half; a.eps = eps;
   // Few tokens: four waves' worth of heads per workgroup, for many workgroups; many tokens: all heads of a token.
   const int heads = nq + 2 * nkv;
   const int lph = d / VK_VEC;          // lanes per head in the kernel with 16-byte accesses
   const bool vec = (d == 64 || d == 128 || d == 256) && lph <= 64 && (cos_t == nullptr || 2 * rot_half == d) &&
                    row_stride % VK_VEC == 0 && ((uintptr_t)qkv % 16) == 0 && (q_out == nullptr || (uintptr_t)q_out % 16 == 0) &&
-                   (kc == nullptr || (uintptr_t)kc % 16 == 0) && (cos_t == nullptr || ((uintptr_t)cos_t % 16 == 0 && (uintptr_t)sin_t % 16 == 0));
+                   (kc == nullptr || (uintptr_t)kc % 16 == 0) && (bias == nullptr || (uintptr_t)bias % 16 == 0) && (cos_t == nullptr || ((uintptr_t)cos_t % 16 == 0 && (uintptr_t)sin_t % 16 == 0));
   if (vec) {
     const int hpw = 64 / lph, per_wg = 4 * hpw;
     const int per_wave = T >= 512 ? (heads + per_wg - 1) / per_wg : 1;
@@ -246,6 +254,24 @@ int vk_qkv_post(const elem_t* qkv, int64_t row_stride, elem_t* q_out, elem_t* kc
   const int per_wave = T >= 512 ? (heads + 3) / 4 : 1;
   qkv_post_kernel<<<dim3(T, (heads + 4 * per_wave - 1) / (4 * per_wave)), 256, 0, st>>>(a, per_wave);
   return vk_check_launch("qkv_post");
+}
+
+int vk_qkv_post(const elem_t* qkv, int64_t row_stride, elem_t* q_out, elem_t* kc, elem_t* vc, const void* q_w,
+                const void* k_w, int w_is_f32, const elem_t* cos_t, const elem_t* sin_t, int rot_half,
+                const int32_t* positions, const int32_t* slots, int T, int nq, int nkv, int d, int P, float eps,
+                hipStream_t st) {
+  return qkv_post_launch(qkv, row_stride, q_out, kc, vc, q_w, k_w, w_is_f32, cos_t, sin_t, rot_half, positions, slots, T, nq, nkv, d, P, eps,
+                         nullptr, st);
+}
+
+// The same with a bias [(nq + 2 nkv) d] that is added to every row before anything else, as a projection with a bias
+// would have left it.
+int vk_qkv_post_bias(const elem_t* qkv, int64_t row_stride, elem_t* q_out, elem_t* kc, elem_t* vc, const void* q_w,
+                     const void* k_w, int w_is_f32, const elem_t* cos_t, const elem_t* sin_t, int rot_half,
+                     const int32_t* positions, const int32_t* slots, int T, int nq, int nkv, int d, int P, float eps,
+                     const elem_t* bias, hipStream_t st) {
+  return qkv_post_launch(qkv, row_stride, q_out, kc, vc, q_w, k_w, w_is_f32, cos_t, sin_t, rot_half, positions, slots, T, nq, nkv, d, P, eps,
+                         bias, st);
 }
 
 }  // extern "C"

@@ -1,0 +1,158 @@
+// Kernels for a residual stream that is kept in 32-bit whatever the element type: the embedding with sinusoidal
+// positions added, the norm that reads the stream and writes elements, the norm of a sublayer's output that is
+// scaled and added to the stream, the weighted sum of the stream's earlier states, a row gather, and the cap of
+// the logits.
+//
+// Norms here are y = x * rsqrt(mean(x^2) + eps) * (offset + w): offset 1 is the weight stored around zero, offset 0
+// the plain weight.  One workgroup per row; thread t owns the elements t, t + 256, ... of the row, its partial sum
+// runs over them in that order, a wave butterfly follows and the four wave sums are added in wave order, so the
+// order depends on the row's length alone.
+#include "common.h"
+#include "vec.h"
+
+#define STREAM_THREADS 256
+
+__device__ __forceinline__ float stream_block_sum(float v, float* red) {
+  v = wave_sum_xor(v);
+  const int wave = threadIdx.x >> 6;
+  if ((threadIdx.x & 63) == 0) red[wave] = v;
+  __syncthreads();
+  float s = red[0];
+  s = s + red[1];
+  s = s + red[2];
+  s = s + red[3];
+  return s;
+}
+
+// out[t, 2i] = table[id, 2i] + sin(p * f[i]); out[t, 2i + 1] = table[id, 2i + 1] + cos(p * f[i]); angles in 32-bit.
+__global__ __launch_bounds__(STREAM_THREADS) void embed_sinusoid_kernel(float* __restrict__ out, const elem_t* __restrict__ table,
+                                                                        const int32_t* __restrict__ ids,
+                                                                        const int32_t* __restrict__ positions,
+                                                                        const float* __restrict__ inv_freq, int H) {
+  const int t = blockIdx.x;
+  const elem_t* src = table + (int64_t)ids[t] * H;
+  const float p = (float)positions[t];
+  float* dst = out + (int64_t)t * H;
+  for (int c = threadIdx.x; c < H; c += blockDim.x) {
+    const float angle = p * inv_freq[c >> 1];
+    dst[c] = to_f32(src[c]) + ((c & 1) ? cosf(angle) : sinf(angle));
+  }
+}
+
+template <bool IN_F32>
+__device__ __forceinline__ float stream_load(const void* x, int64_t i) {
+  return IN_F32 ? static_cast<const float*>(x)[i] : to_f32(static_cast<const elem_t*>(x)[i]);
+}
+
+// out (elements) = norm of a row of the stream (IN_F32) or of elements.
+template <bool IN_F32>
+__global__ __launch_bounds__(STREAM_THREADS) void stream_norm_kernel(elem_t* __restrict__ out, const void* __restrict__ x,
+                                                                     const void* __restrict__ w, int w_is_f32, int H, float eps,
+                                                                     float offset) {
+  __shared__ float red[4];
+  const int64_t base = (int64_t)blockIdx.x * H;
+  float part = 0.f;
+  for (int c = threadIdx.x; c < H; c += STREAM_THREADS) {
+    const float v = stream_load<IN_F32>(x, base + c);
+    part = part + v * v;
+  }
+  const float rr = rsqrtf(stream_block_sum(part, red) / (float)H + eps);
+  for (int c = threadIdx.x; c < H; c += STREAM_THREADS) {
+    const float v = stream_load<IN_F32>(x, base + c);
+    out[base + c] = from_f32<elem_t>((v * rr) * (offset + load_weight(w, w_is_f32, c)));
+  }
+}
+
+// out = base + mult * norm(y), rows of the stream; out may be base.
+__global__ __launch_bounds__(STREAM_THREADS) void stream_norm_add_kernel(float* out, const float* base_rows, const elem_t* __restrict__ y,
+                                                                         const void* __restrict__ w, int w_is_f32, int H, float eps,
+                                                                         float offset, float mult) {
+  __shared__ float red[4];
+  const int64_t base = (int64_t)blockIdx.x * H;
+  float part = 0.f;
+  for (int c = threadIdx.x; c < H; c += STREAM_THREADS) {
+    const float v = to_f32(y[base + c]);
+    part = part + v * v;
+  }
+  const float rr = rsqrtf(stream_block_sum(part, red) / (float)H + eps);
+  for (int c = threadIdx.x; c < H; c += STREAM_THREADS) {
+    const float v = to_f32(y[base + c]);
+    const float n = (v * rr) * (offset + load_weight(w, w_is_f32, c));
+    out[base + c] = base_rows[base + c] + mult * n;
+  }
+}
+
+// out[e] = sum over j < n of coef[j] * states[j * stride + e], added in ascending j from zero.
+__global__ __launch_bounds__(256) void stream_mix_kernel(float* __restrict__ out, const float* __restrict__ states, int64_t stride,
+                                                         const void* __restrict__ coef, int coef_is_f32, int n, int64_t numel) {
+  const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= numel) return;
+  float acc = 0.f;
+  for (int j = 0; j < n; ++j) acc = acc + load_weight(coef, coef_is_f32, j) * states[j * stride + e];
+  out[e] = acc;
+}
+
+__global__ __launch_bounds__(256) void gather_rows_f32_kernel(float* __restrict__ out, const float* __restrict__ x,
+                                                              const int32_t* __restrict__ rows, int H) {
+  const float* src = x + (int64_t)rows[blockIdx.x] * H;
+  float* dst = out + (int64_t)blockIdx.x * H;
+  for (int c = threadIdx.x; c < H; c += blockDim.x) dst[c] = src[c];
+}
+
+// x <- cap * tanh(x / cap), in 32-bit, stored as elements.
+__global__ __launch_bounds__(256) void softcap_kernel(elem_t* x, float cap, int64_t n) {
+  const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e < n) x[e] = from_f32<elem_t>(cap * tanhf(to_f32(x[e]) / cap));
+}
+
+extern "C" {
+
+int vk_embed_sinusoid(float* out, const elem_t* table, const int32_t* ids, const int32_t* positions, const float* inv_freq, int T,
+                      int H, int V, hipStream_t st) {
+  VK_REQUIRE(T >= 0 && H > 0 && H % 2 == 0 && V > 0, "sinusoidal embedding: bad sizes T=%d H=%d V=%d (the width must be even)", T, H, V);
+  if (T == 0) return 0;
+  embed_sinusoid_kernel<<<T, STREAM_THREADS, 0, st>>>(out, table, ids, positions, inv_freq, H);
+  return vk_check_launch("sinusoidal embedding");
+}
+
+// x: rows of floats (x_is_f32) or of elements; out: elements.
+int vk_stream_norm(elem_t* out, const void* x, int x_is_f32, const void* w, int w_is_f32, int rows, int H, float eps, float offset,
+                   hipStream_t st) {
+  VK_REQUIRE(rows >= 0 && H > 0 && eps >= 0.f, "stream norm: bad sizes rows=%d H=%d", rows, H);
+  if (rows == 0) return 0;
+  if (x_is_f32) stream_norm_kernel<true><<<rows, STREAM_THREADS, 0, st>>>(out, x, w, w_is_f32, H, eps, offset);
+  else stream_norm_kernel<false><<<rows, STREAM_THREADS, 0, st>>>(out, x, w, w_is_f32, H, eps, offset);
+  return vk_check_launch("stream norm");
+}
+
+int vk_stream_norm_add(float* out, const float* base, const elem_t* y, const void* w, int w_is_f32, int rows, int H, float eps,
+                       float offset, float mult, hipStream_t st) {
+  VK_REQUIRE(rows >= 0 && H > 0 && eps >= 0.f, "stream norm-add: bad sizes rows=%d H=%d", rows, H);
+  if (rows == 0) return 0;
+  stream_norm_add_kernel<<<rows, STREAM_THREADS, 0, st>>>(out, base, y, w, w_is_f32, H, eps, offset, mult);
+  return vk_check_launch("stream norm-add");
+}
+
+int vk_stream_mix(float* out, const float* states, int64_t stride, const void* coef, int coef_is_f32, int n, int64_t numel,
+                  hipStream_t st) {
+  VK_REQUIRE(n > 0 && numel >= 0 && stride >= numel, "stream mix: bad sizes n=%d numel=%lld stride=%lld", n, (long long)numel, (long long)stride);
+  if (numel == 0) return 0;
+  stream_mix_kernel<<<(unsigned)((numel + 255) / 256), 256, 0, st>>>(out, states, stride, coef, coef_is_f32, n, numel);
+  return vk_check_launch("stream mix");
+}
+
+int vk_gather_rows_f32(float* out, const float* x, const int32_t* rows, int R, int H, hipStream_t st) {
+  VK_REQUIRE(R >= 0 && H > 0, "gather_rows: bad sizes R=%d H=%d", R, H);
+  if (R == 0) return 0;
+  gather_rows_f32_kernel<<<R, 256, 0, st>>>(out, x, rows, H);
+  return vk_check_launch("gather_rows (32-bit)");
+}
+
+int vk_softcap(elem_t* x, float cap, int64_t n, hipStream_t st) {
+  VK_REQUIRE(cap > 0.f && n >= 0, "softcap: the cap must be positive");
+  if (n == 0) return 0;
+  softcap_kernel<<<(unsigned)((n + 255) / 256), 256, 0, st>>>(x, cap, n);
+  return vk_check_launch("softcap");
+}
+
+}  // extern "C"
