@@ -6,6 +6,7 @@
     python bench.py --workload mixed14b     # Qwen3-14B shape: 32 prompts of 128 to 4,096 tokens, prefill in portions beside decoding
     python bench.py --workload prefix32b    # Qwen3-32B shape: 64 requests at context 8,192 that share a 1,024-token prefix
     python bench.py --workload aligned      # the reference's aligned phases: batch 4, cached contexts 0 to 16K, 256 new tokens / 127 decode steps
+    python bench.py --workload tezinex      # the Tezinex design at three layer sizes beside the Qwen3 decoder at equal size: prefill and decode
 
 A step is one decode step of the engine (plan, forward, sample, commit) for a
 batch of B requests whose prompts of 2,048 random tokens were prefilled through
@@ -85,7 +86,7 @@ def main() -> int:
     ap.add_argument("--no-other-shapes", action="store_true", help="skip the 14B and 32B workloads that the default record holds as points")
     ap.add_argument("--prompt-tokens", type=int, default=PROMPT_TOKENS,
                     help="context length of the decode measurement (the prefill figure is always of 2,048 tokens)")
-    ap.add_argument("--workload", default="decode8b", choices=["decode8b", "mixed14b", "prefix32b", "aligned"])
+    ap.add_argument("--workload", default="decode8b", choices=["decode8b", "mixed14b", "prefix32b", "aligned", "tezinex"])
     ap.add_argument("--engine", default="native", choices=["native", "python"],
                     help="which engine every figure is measured through: the native one (vosti_amd.engine.NativeEngine) or the "
                          "Python step function over the same kernels, cache manager and scheduler")
@@ -107,6 +108,9 @@ def main() -> int:
 
     if args.workload == "aligned":
         print(json.dumps(aligned_workload(args)), flush=True)
+        return 0
+    if args.workload == "tezinex":
+        print(json.dumps(tezinex_workload(args)), flush=True)
         return 0
     if args.workload != "decode8b":
         print(json.dumps(other_workload(args)), flush=True)
@@ -500,6 +504,99 @@ def aligned_workload(args) -> dict:
             "roofline": {"bound": "hbm", "achieved": round(read / step_s / 1e9, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": round(read / step_s / 1e9 / HBM_PEAK_GBS, 4)},
             "points": points, "intervals": detail}
+
+
+# Layer sizes for --workload tezinex: (width, q heads, kv heads, feed-forward).  Heads are 128 wide, as in the Qwen3 shapes.
+TEZINEX_SIZES = {"1k": (1024, 8, 2, 3072), "2k": (2048, 16, 4, 6144), "4k": (4096, 32, 8, 12288)}
+
+
+def tezinex_config(width, heads, kv_heads, ff, layers, vocab):
+    """Delta, attention, attention on the keys of the one before, delta, ...: every layer with a feed-forward, so that
+    a layer's matrix work is that of a Qwen3 layer of the same sizes."""
+    def attention(kv_from=None):
+        m = {"dim": 128, "vdim": 128, "heads": heads, "kv_heads": kv_heads, "mask": {"size": 1024, "keep_first": 16},
+             "scale": 128 ** -0.5, "softcap": 30.0}
+        if kv_from is not None:
+            m["kv_from"] = kv_from
+        return {"type": "attention", "mixer": m, "mlp": {"kind": "dense", "ff": ff}}
+    delta = {"type": "channel_delta", "mixer": {"dim": 128, "vdim": 128, "heads": heads, "kv_heads": heads, "conv": 4},
+             "mlp": {"kind": "dense", "ff": ff}}
+    out = []
+    for i in range(layers):
+        kind = i % 4
+        out.append(delta if kind in (0, 3) else attention(i - 1 if kind == 2 else None))
+    return {"architecture": "Tezinex", "layers": out, "logit_softcap": 30.0, "norm": {"eps": 1e-6}, "residual_mult": 0.7, "vocab": vocab,
+            "width": width}
+
+
+def tezinex_workload(args) -> dict:
+    """Prefill of one prompt and decoding at a fixed batch for the Tezinex design at three layer sizes, each beside the
+    Qwen3 decoder with the same width, heads, feed-forward, layers and vocabulary (random weights, the native engine)."""
+    import tempfile
+    from vosti_amd.engine import NativeEngine
+    from vosti_amd.sampling import SamplingParams
+
+    layers = args.layers if args.layers is not None else 8
+    batch = args.batch if args.batch is not None else 8
+    prompt_tokens, vocab, page = args.prompt_tokens, 32768, 64
+    rng = random.Random(2)
+    record = {"metric": "decode_tokens_per_s", "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+              "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
+              "data": "synthetic: seeded random token prompts, seeded random weights", "sizes": {},
+              "config": {"model": "Tezinex (delta, attention, shared-key attention, delta, ...) beside Qwen3 at equal size", "layers": layers,
+                         "global_batch": batch, "seq_len": prompt_tokens, "vocab_size": vocab, "parallelism": "single GPU",
+                         "graphs": bool(args.graphs)}}
+
+    def measure(config: dict) -> dict:
+        with tempfile.TemporaryDirectory() as d:
+            with open(os.path.join(d, "config.json"), "w") as f:
+                json.dump(config, f)
+            pages = (batch + 1) * -(-(prompt_tokens + args.steps + args.warmup + 2) // page) + 4
+            eng = NativeEngine(d, dtype=args.dtype, random_weights_seed=0, num_pages=pages, page_size=page, max_num_seqs=batch,
+                               max_num_batched_tokens=max(prompt_tokens, 256), enable_prefix_cache=False, graphs=bool(args.graphs))
+            prompt = lambda: [rng.randrange(vocab) for _ in range(prompt_tokens)]
+            # Prefill: a whole prompt in one step, the median of five after one untimed.
+            times = []
+            for rep in range(6):
+                eng.add_request(prompt(), SamplingParams(max_tokens=1, ignore_eos=True))
+                eng.synchronize()
+                t0 = time.perf_counter()
+                while eng.has_unfinished():
+                    eng.step()
+                eng.synchronize()
+                times.append(time.perf_counter() - t0)
+            prefill_s = sorted(times[1:])[2]
+            # Decode: `batch` requests at that context, warm-up steps, then the timed ones.
+            for _ in range(batch):
+                eng.add_request(prompt(), SamplingParams(max_tokens=args.steps + args.warmup + 1, ignore_eos=True))
+            emitted = 0
+            while emitted < batch:                                   # the prompts enter one a step
+                emitted += len(eng.step())
+            for _ in range(args.warmup):
+                eng.step()
+            eng.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(args.steps):
+                eng.step()
+            eng.synchronize()
+            step_s = (time.perf_counter() - t0) / args.steps
+            while eng.has_unfinished():
+                eng.step()
+            return {"prefill_ms": round(prefill_s * 1e3, 3), "prefill_tokens_per_s": round(prompt_tokens / prefill_s, 1),
+                    "decode_ms_per_step": round(step_s * 1e3, 4), "decode_tokens_per_s": round(batch / step_s, 1)}
+
+    for name, (width, heads, kv_heads, ff) in TEZINEX_SIZES.items():
+        print(f"bench.py: tezinex: width {width}, {layers} layers", file=sys.stderr, flush=True)
+        tez = measure(tezinex_config(width, heads, kv_heads, ff, layers, vocab))
+        qwen = measure(dict(QWEN3_8B, architectures=["Qwen3ForCausalLM"], vocab_size=vocab, hidden_size=width, intermediate_size=ff,
+                            num_hidden_layers=layers, num_attention_heads=heads, num_key_value_heads=kv_heads, tie_word_embeddings=True))
+        record["sizes"][name] = {"width": width, "q_heads": heads, "kv_heads": kv_heads, "ff": ff, "tezinex": tez, "qwen3": qwen,
+                                 "decode_ratio": round(tez["decode_tokens_per_s"] / qwen["decode_tokens_per_s"], 3),
+                                 "prefill_ratio": round(tez["prefill_tokens_per_s"] / qwen["prefill_tokens_per_s"], 3)}
+    last = record["sizes"]["4k"]["tezinex"]
+    record["value"] = last["decode_tokens_per_s"]
+    record["ms_per_step"] = last["decode_ms_per_step"]
+    return record
 
 
 def other_workload(args) -> dict:

@@ -8,7 +8,7 @@ from ctypes import POINTER, c_char_p, c_double, c_int, c_int32, c_int64, c_uint6
 
 from ..kernels import build
 
-ABI_VERSION = 8
+ABI_VERSION = 9
 _LIB = None
 
 
@@ -28,6 +28,7 @@ def host_lib():
         fn.restype, fn.argtypes = restype, list(args)
 
     sig("vh_cache_create", P, I, I, POINTER(c_int), POINTER(c_int), I, I)
+    sig("vh_cache_create_kept", P, I, I, POINTER(c_int), POINTER(c_int), POINTER(c_int), I, I)
     sig("vh_cache_destroy", None, P)
     sig("vh_cache_add_request", I, P, U, PI, I, POINTER(c_int))
     sig("vh_cache_reserve", I, P, U, I)

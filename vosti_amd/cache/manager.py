@@ -30,6 +30,7 @@ class OutOfPages(CacheError):
 class GroupSpec:
     window: int      # 0: all keys
     num_pages: int
+    keep_first: int = 0   # with a window: the pages of a request's first keep_first keys are never given back
 
 
 class CacheManager:
@@ -40,7 +41,8 @@ class CacheManager:
         self.page_size, self.groups, self.num_slots = page_size, list(groups), num_slots
         windows = (c_int * len(groups))(*[g.window for g in groups])
         pages = (c_int * len(groups))(*[g.num_pages for g in groups])
-        self._h = self._lib.vh_cache_create(page_size, len(groups), windows, pages, num_slots, 1 if prefix_cache else 0)
+        keeps = (c_int * len(groups))(*[g.keep_first for g in groups])
+        self._h = self._lib.vh_cache_create_kept(page_size, len(groups), windows, keeps, pages, num_slots, 1 if prefix_cache else 0)
         if not self._h:
             raise CacheError("bad cache geometry")
         self.prefix_cache = prefix_cache and all(g.window == 0 for g in groups)

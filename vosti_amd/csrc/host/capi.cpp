@@ -22,7 +22,7 @@ struct SchedulerHandle {
 
 extern "C" {
 
-int vh_abi_version(void) { return 8; }
+int vh_abi_version(void) { return 9; }
 
 // ------------------------------------------------------------ cache manager
 void* vh_cache_create(int page_size, int n_groups, const int* windows, const int* num_pages, int num_slots,
@@ -32,6 +32,17 @@ void* vh_cache_create(int page_size, int n_groups, const int* windows, const int
   for (int g = 0; g < n_groups; ++g) {
     if (windows[g] < 0 || num_pages[g] < 0) return nullptr;
     groups.push_back(GroupSpec{windows[g], num_pages[g]});
+  }
+  return new CacheManager(page_size, groups, num_slots, prefix_cache != 0);
+}
+// The same with the number of first keys that every windowed group keeps for good (0 for a group of all keys).
+void* vh_cache_create_kept(int page_size, int n_groups, const int* windows, const int* keep_first, const int* num_pages, int num_slots,
+                           int prefix_cache) {
+  if (page_size <= 0 || n_groups <= 0 || num_slots < 0) return nullptr;
+  std::vector<GroupSpec> groups;
+  for (int g = 0; g < n_groups; ++g) {
+    if (windows[g] < 0 || num_pages[g] < 0 || keep_first[g] < 0) return nullptr;
+    groups.push_back(GroupSpec{windows[g], num_pages[g], keep_first[g]});
   }
   return new CacheManager(page_size, groups, num_slots, prefix_cache != 0);
 }
