@@ -87,6 +87,8 @@ def main() -> int:
     ap.add_argument("--prompt-tokens", type=int, default=PROMPT_TOKENS,
                     help="context length of the decode measurement (the prefill figure is always of 2,048 tokens)")
     ap.add_argument("--workload", default="decode8b", choices=["decode8b", "mixed14b", "prefix32b", "aligned", "tezinex"])
+    ap.add_argument("--sizes", default=",".join(["1k", "2k", "4k"]), help="which layer sizes --workload tezinex measures (1k, 2k, 4k)")
+    ap.add_argument("--only-design", default="", choices=["", "tezinex", "qwen3"], help="--workload tezinex: measure one of the two designs only")
     ap.add_argument("--engine", default="native", choices=["native", "python"],
                     help="which engine every figure is measured through: the native one (vosti_amd.engine.NativeEngine) or the "
                          "Python step function over the same kernels, cache manager and scheduler")
@@ -585,17 +587,23 @@ def tezinex_workload(args) -> dict:
             return {"prefill_ms": round(prefill_s * 1e3, 3), "prefill_tokens_per_s": round(prompt_tokens / prefill_s, 1),
                     "decode_ms_per_step": round(step_s * 1e3, 4), "decode_tokens_per_s": round(batch / step_s, 1)}
 
-    for name, (width, heads, kv_heads, ff) in TEZINEX_SIZES.items():
+    for name in [n for n in args.sizes.split(",") if n]:
+        width, heads, kv_heads, ff = TEZINEX_SIZES[name]
         print(f"bench.py: tezinex: width {width}, {layers} layers", file=sys.stderr, flush=True)
-        tez = measure(tezinex_config(width, heads, kv_heads, ff, layers, vocab))
-        qwen = measure(dict(QWEN3_8B, architectures=["Qwen3ForCausalLM"], vocab_size=vocab, hidden_size=width, intermediate_size=ff,
-                            num_hidden_layers=layers, num_attention_heads=heads, num_key_value_heads=kv_heads, tie_word_embeddings=True))
-        record["sizes"][name] = {"width": width, "q_heads": heads, "kv_heads": kv_heads, "ff": ff, "tezinex": tez, "qwen3": qwen,
-                                 "decode_ratio": round(tez["decode_tokens_per_s"] / qwen["decode_tokens_per_s"], 3),
-                                 "prefill_ratio": round(tez["prefill_tokens_per_s"] / qwen["prefill_tokens_per_s"], 3)}
-    last = record["sizes"]["4k"]["tezinex"]
-    record["value"] = last["decode_tokens_per_s"]
-    record["ms_per_step"] = last["decode_ms_per_step"]
+        point = {"width": width, "q_heads": heads, "kv_heads": kv_heads, "ff": ff}
+        if args.only_design != "qwen3":
+            point["tezinex"] = measure(tezinex_config(width, heads, kv_heads, ff, layers, vocab))
+        if args.only_design != "tezinex":
+            point["qwen3"] = measure(dict(QWEN3_8B, architectures=["Qwen3ForCausalLM"], vocab_size=vocab, hidden_size=width, intermediate_size=ff,
+                                          num_hidden_layers=layers, num_attention_heads=heads, num_key_value_heads=kv_heads,
+                                          tie_word_embeddings=True))
+        if "tezinex" in point and "qwen3" in point:
+            point["decode_ratio"] = round(point["tezinex"]["decode_tokens_per_s"] / point["qwen3"]["decode_tokens_per_s"], 3)
+            point["prefill_ratio"] = round(point["tezinex"]["prefill_tokens_per_s"] / point["qwen3"]["prefill_tokens_per_s"], 3)
+        record["sizes"][name] = point
+        last = point.get("tezinex") or point["qwen3"]
+        record["value"] = last["decode_tokens_per_s"]
+        record["ms_per_step"] = last["decode_ms_per_step"]
     return record
 
 

@@ -7,9 +7,9 @@
 // so that the read-out sees the token's own write.  g = exp(-exp(A_log) * softplus(a + dt_bias)), beta = sigmoid(b).
 // Everything here is 32-bit; the projections that feed it (a, b, the convolutions' inputs) arrive as elements.
 //
-// A sequence's tokens are walked in order by one wave per (sequence, head, block of value columns), so the sums of a
-// token do not depend on how the sequence was cut into steps or on what else is in the batch: the state that a step
-// leaves in memory is the state the next step starts from, bit for bit.
+// A sequence's tokens are walked in order by one workgroup per (sequence, head, block of value columns), so the sums
+// of a token do not depend on how the sequence was cut into steps or on what else is in the batch: the state that a
+// step leaves in memory is the state the next step starts from, bit for bit.
 #include "common.h"
 #include "vec.h"
 
@@ -89,64 +89,170 @@ __global__ __launch_bounds__(256) void delta_decay_kernel(float* __restrict__ g,
   g[e] = expf(-expf(load_weight(A_log, w_is_f32, col / d)) * sp);
 }
 
-// The recurrence.  A wave takes 64 / R value columns of one (sequence, head); a column's state is spread over R
-// neighbouring lanes, lane r of them holding the key channels r, r + R, ... (DR of them at most) in registers.
-// The two sums of a token run over a lane's channels in ascending order and then as a butterfly over the R lanes.
-template <int DR>
-__global__ __launch_bounds__(64) void delta_rule_kernel(float* __restrict__ out, const float* __restrict__ qkv, int64_t ld, int q_col,
-                                                        int k_col, int v_col, const float* __restrict__ decay, const elem_t* __restrict__ b,
-                                                        int64_t ldb, float* state, int64_t state_stride,
-                                                        const int32_t* __restrict__ cu_q, const int32_t* __restrict__ positions,
-                                                        const int32_t* __restrict__ slots, int H, int G, int d, int dv, int R) {
+// The recurrence.  A workgroup of four waves takes 4 * 64 / R value columns of one (sequence, head); a column's state
+// is spread over R neighbouring lanes, lane r of them holding the key channels 16 r .. 16 r + 15 in registers.  The
+// inputs of a chunk of tokens (q, k and the decays of the head, the columns' v, beta) are brought into LDS by the whole
+// workgroup, the next chunk's while this one is computed (global memory -> registers before the chunk's work, registers
+// -> the other LDS buffer after it, one barrier a chunk), so that the walk over the tokens waits for LDS only.  The two
+// sums of a token run over a lane's channels in ascending order and then as a butterfly over the R lanes, whatever the
+// chunks are: a token's arithmetic does not know where a step was cut.  In memory a head's state is [vdim][dim], so
+// that a lane's channels are 64 consecutive bytes and a wave's loads are whole lines.
+#define RULE_DR 16
+#define RULE_THREADS 256
+
+template <int R>
+struct RuleShape {
+  static constexpr int DMAX = RULE_DR * R;                       // key channels this instance holds
+  static constexpr int TC = 2048 / DMAX < 16 ? 2048 / DMAX : 16; // tokens a chunk
+  static constexpr int CB = 4 * 64 / R;                          // value columns a workgroup
+  static constexpr int BUF = (TC * (3 * DMAX + CB + 1) + 3) / 4 * 4;   // floats of one LDS buffer: k, q, g, v, beta
+  static constexpr int NI = (TC * DMAX + RULE_THREADS - 1) / RULE_THREADS;
+  static constexpr int NV = (TC * CB + RULE_THREADS - 1) / RULE_THREADS;
+};
+
+template <int R>
+__global__ __launch_bounds__(RULE_THREADS) void delta_rule_kernel(float* __restrict__ out, const float* __restrict__ qkv, int64_t ld, int q_col,
+                                                                  int k_col, int v_col, const float* __restrict__ decay,
+                                                                  const elem_t* __restrict__ b, int64_t ldb, float* state, int64_t state_stride,
+                                                                  const int32_t* __restrict__ cu_q, const int32_t* __restrict__ positions,
+                                                                  const int32_t* __restrict__ slots, int H, int G, int d, int dv) {
+  using Sh = RuleShape<R>;
+  constexpr int DR = RULE_DR, DMAX = Sh::DMAX, TC = Sh::TC, CB = Sh::CB;
+  __shared__ __attribute__((aligned(16))) float smem[2 * Sh::BUF];
   const int s = blockIdx.x, h = blockIdx.y;
-  const int lane = threadIdx.x;
-  const int r = lane % R, cols = 64 / R;
-  const int col = blockIdx.z * cols + lane / R;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int r = lane % R;
+  const int col_in_block = wave * (64 / R) + lane / R;
+  const int col = blockIdx.z * CB + col_in_block;
   const bool col_ok = col < dv;
   const int g = h / (H / G);
   const int first = cu_q[s], n = cu_q[s + 1] - first;
   const bool fresh = positions[first] == 0;
-  float* S_mem = state + (int64_t)slots[s] * state_stride + (int64_t)h * d * dv;
+  float* S_mem = state + (int64_t)slots[s] * state_stride + ((int64_t)h * dv + (col_ok ? col : 0)) * d + r * DR;
+  const bool rows_vec = d % 4 == 0 && (((uintptr_t)S_mem) & 15) == 0;
   float S[DR];
 #pragma unroll
-  for (int i = 0; i < DR; ++i) {
-    const int row = r + i * R;
-    S[i] = (!fresh && col_ok && row < d) ? S_mem[(int64_t)row * dv + col] : 0.f;
-  }
-  for (int i0 = 0; i0 < n; ++i0) {
-    const int64_t t = first + i0;
-    const float* qrow = qkv + t * ld + q_col + (int64_t)g * d;
-    const float* krow = qkv + t * ld + k_col + (int64_t)g * d;
-    const float* grow = decay + (t * H + h) * d;
-    const float v = col_ok ? qkv[t * ld + v_col + (int64_t)h * dv + col] : 0.f;
-    const float beta = sigmoid_f(to_f32(b[t * ldb + h]));
-    float kk[DR], qq[DR];
-    float dot = 0.f;
+  for (int i = 0; i < DR; ++i) S[i] = 0.f;
+  if (!fresh && col_ok) {
+    if (rows_vec) {
 #pragma unroll
-    for (int i = 0; i < DR; ++i) {
-      const int row = r + i * R;
-      const bool ok = row < d;
-      kk[i] = ok ? krow[row] : 0.f;
-      qq[i] = ok ? qrow[row] : 0.f;
-      const float gg = ok ? grow[row] : 1.f;
-      S[i] = S[i] * gg;
-      dot = dot + S[i] * kk[i];
+      for (int i = 0; i < DR; i += 4) {
+        if (r * DR + i < d) {
+          const f32x4 v4 = *reinterpret_cast<const f32x4*>(S_mem + i);
+          S[i] = v4.x; S[i + 1] = v4.y; S[i + 2] = v4.z; S[i + 3] = v4.w;
+        }
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < DR; ++i)
+        if (r * DR + i < d) S[i] = S_mem[i];
     }
-    for (int m = 1; m < R; m <<= 1) dot = dot + __shfl_xor(dot, m, VK_WAVE);
-    const float u = beta * (v - dot);
-    float o = 0.f;
-#pragma unroll
-    for (int i = 0; i < DR; ++i) {
-      S[i] = S[i] + kk[i] * u;
-      o = o + S[i] * qq[i];
-    }
-    for (int m = 1; m < R; m <<= 1) o = o + __shfl_xor(o, m, VK_WAVE);
-    if (col_ok && r == 0) out[(t * H + h) * dv + col] = o;
   }
+
+  // What this thread brings in of a chunk: elements e = tid, tid + 256, ... of the chunk's [TC][DMAX] tiles of k, q and
+  // the decays, and of its [TC][CB] tile of v; beta by the first TC threads.  Channels beyond d read as k = q = 0, g = 1.
+  float pk[Sh::NI], pq[Sh::NI], pg[Sh::NI], pv[Sh::NV], pb = 0.f;
+  auto fetch = [&](int chunk) {
+    const int t0 = chunk * TC;
 #pragma unroll
-  for (int i = 0; i < DR; ++i) {
-    const int row = r + i * R;
-    if (col_ok && row < d) S_mem[(int64_t)row * dv + col] = S[i];
+    for (int it = 0; it < Sh::NI; ++it) {
+      const int e = tid + it * RULE_THREADS;
+      const int tok = e / DMAX, c = e - tok * DMAX;
+      const bool ok = e < TC * DMAX && t0 + tok < n && c < d;
+      const int64_t t = first + t0 + (ok ? tok : 0);
+      const int cc = ok ? c : 0;
+      const float kv = qkv[t * ld + k_col + (int64_t)g * d + cc], qv = qkv[t * ld + q_col + (int64_t)g * d + cc];
+      const float gv = decay[(t * H + h) * d + cc];
+      pk[it] = ok ? kv : 0.f;
+      pq[it] = ok ? qv : 0.f;
+      pg[it] = ok ? gv : 1.f;
+    }
+#pragma unroll
+    for (int it = 0; it < Sh::NV; ++it) {
+      const int e = tid + it * RULE_THREADS;
+      const int tok = e / CB, c = e - tok * CB;
+      const bool ok = e < TC * CB && t0 + tok < n && blockIdx.z * CB + c < dv;
+      const int64_t t = first + t0 + (ok ? tok : 0);
+      const float vv = qkv[t * ld + v_col + (int64_t)h * dv + (ok ? blockIdx.z * CB + c : 0)];
+      pv[it] = ok ? vv : 0.f;
+    }
+    if (tid < TC) {
+      const bool ok = t0 + tid < n;
+      const float bb = to_f32(b[(int64_t)(first + t0 + (ok ? tid : 0)) * ldb + h]);
+      pb = ok ? sigmoid_f(bb) : 0.f;
+    }
+  };
+  auto stage = [&](int buffer) {
+    float* base = smem + buffer * Sh::BUF;
+#pragma unroll
+    for (int it = 0; it < Sh::NI; ++it) {
+      const int e = tid + it * RULE_THREADS;
+      if (e < TC * DMAX) {
+        base[e] = pk[it];
+        base[TC * DMAX + e] = pq[it];
+        base[2 * TC * DMAX + e] = pg[it];
+      }
+    }
+#pragma unroll
+    for (int it = 0; it < Sh::NV; ++it) {
+      const int e = tid + it * RULE_THREADS;
+      if (e < TC * CB) base[3 * TC * DMAX + e] = pv[it];
+    }
+    if (tid < TC) base[3 * TC * DMAX + TC * CB + tid] = pb;
+  };
+
+  const int chunks = (n + TC - 1) / TC;
+  fetch(0);
+  stage(0);
+  __syncthreads();
+  for (int chunk = 0; chunk < chunks; ++chunk) {
+    const float* base = smem + (chunk & 1) * Sh::BUF;
+    if (chunk + 1 < chunks) fetch(chunk + 1);
+    const int here = min(TC, n - chunk * TC);
+    for (int tok = 0; tok < here; ++tok) {
+      const float* kr = base + tok * DMAX + r * DR;
+      const float* qr = kr + TC * DMAX;
+      const float* gr = qr + TC * DMAX;
+      const float v = base[3 * TC * DMAX + tok * CB + col_in_block];
+      const float beta = base[3 * TC * DMAX + TC * CB + tok];
+      float kk[DR], qq[DR];
+      float dot = 0.f;
+#pragma unroll
+      for (int i = 0; i < DR; i += 4) {
+        const f32x4 k4 = *reinterpret_cast<const f32x4*>(kr + i), g4 = *reinterpret_cast<const f32x4*>(gr + i);
+        const f32x4 q4 = *reinterpret_cast<const f32x4*>(qr + i);
+        kk[i] = k4.x; kk[i + 1] = k4.y; kk[i + 2] = k4.z; kk[i + 3] = k4.w;
+        qq[i] = q4.x; qq[i + 1] = q4.y; qq[i + 2] = q4.z; qq[i + 3] = q4.w;
+        S[i] = S[i] * g4.x; S[i + 1] = S[i + 1] * g4.y; S[i + 2] = S[i + 2] * g4.z; S[i + 3] = S[i + 3] * g4.w;
+      }
+#pragma unroll
+      for (int i = 0; i < DR; ++i) dot = dot + S[i] * kk[i];
+#pragma unroll
+      for (int m = 1; m < R; m <<= 1) dot = dot + __shfl_xor(dot, m, VK_WAVE);
+      const float u = beta * (v - dot);
+      float o = 0.f;
+#pragma unroll
+      for (int i = 0; i < DR; ++i) {
+        S[i] = S[i] + kk[i] * u;
+        o = o + S[i] * qq[i];
+      }
+#pragma unroll
+      for (int m = 1; m < R; m <<= 1) o = o + __shfl_xor(o, m, VK_WAVE);
+      if (col_ok && r == 0) out[((int64_t)(first + chunk * TC + tok) * H + h) * dv + col] = o;
+    }
+    if (chunk + 1 < chunks) stage((chunk + 1) & 1);
+    __syncthreads();
+  }
+  if (col_ok) {
+    if (rows_vec) {
+#pragma unroll
+      for (int i = 0; i < DR; i += 4)
+        if (r * DR + i < d) *reinterpret_cast<f32x4*>(S_mem + i) = f32x4{S[i], S[i + 1], S[i + 2], S[i + 3]};
+    } else {
+#pragma unroll
+      for (int i = 0; i < DR; ++i)
+        if (r * DR + i < d) S_mem[i] = S[i];
+    }
   }
 }
 
@@ -166,12 +272,10 @@ __global__ __launch_bounds__(64) void delta_out_kernel(elem_t* __restrict__ y, c
 
 extern "C" {
 
-// Lanes that share a value column, for key size d and value size dv: enough that a lane holds 64 channels at most,
-// and more while whole columns' worth of lanes would idle.
-int vk_delta_lanes_per_column(int d, int dv) {
+// Lanes that share a value column for key size d: each holds 16 key channels.
+int vk_delta_lanes_per_column(int d) {
   int R = 1;
-  while (R < 64 && (d + R - 1) / R > 64) R *= 2;
-  while (R < 64 && 64 / R >= 2 * dv && (d + R - 1) / R > 8) R *= 2;
+  while (R < 64 && R * RULE_DR < d) R *= 2;
   return R;
 }
 
@@ -211,23 +315,29 @@ int vk_delta_decay(float* g, const elem_t* a, const void* dt_bias, const void* A
 
 // out [T, H, dv] floats.  qkv: float rows of length ld with q (G heads of d) at q_col, k at k_col, v (H heads of dv) at
 // v_col; decay [T, H, d] floats; b: elements, beta's pre-activation of head h at b[t * ldb + h].  state: per slot,
-// the H states [d, dv] at its start.
+// the H states at its start, each [dv][d].
 int vk_delta_rule(float* out, const float* qkv, int64_t ld, int q_col, int k_col, int v_col, const float* decay, const elem_t* b, int64_t ldb,
                   float* state, int64_t state_stride, const int32_t* cu_q, const int32_t* positions, const int32_t* slots, int S, int H, int G,
                   int d, int dv, hipStream_t st) {
   VK_REQUIRE(S >= 0 && H > 0 && G > 0 && H % G == 0 && d > 0 && dv > 0, "delta rule: bad sizes H=%d G=%d d=%d dv=%d", H, G, d, dv);
-  VK_REQUIRE(d <= 4096, "delta rule: key size %d exceeds 4096", d);
+  VK_REQUIRE(d <= 64 * RULE_DR, "delta rule: key size %d exceeds %d", d, 64 * RULE_DR);
   VK_REQUIRE(state_stride >= (int64_t)H * d * dv, "delta rule: the state is too small");
   if (S == 0) return 0;
-  const int R = vk_delta_lanes_per_column(d, dv);
-  const int per_lane = (d + R - 1) / R, cols = 64 / R;
+  const int R = vk_delta_lanes_per_column(d);
+  const int cols = 4 * 64 / R;
   const dim3 grid(S, H, (dv + cols - 1) / cols);
   VK_REQUIRE(grid.y <= 65535 && grid.z <= 65535, "delta rule: too many heads or columns");
-#define RULE(DR) delta_rule_kernel<DR><<<grid, 64, 0, st>>>(out, qkv, ld, q_col, k_col, v_col, decay, b, ldb, state, state_stride, cu_q, positions, slots, H, G, d, dv, R)
-  if (per_lane <= 8) RULE(8);
-  else if (per_lane <= 16) RULE(16);
-  else if (per_lane <= 32) RULE(32);
-  else RULE(64);
+#define RULE(RR) \
+  delta_rule_kernel<RR><<<grid, RULE_THREADS, 0, st>>>(out, qkv, ld, q_col, k_col, v_col, decay, b, ldb, state, state_stride, cu_q, positions, slots, H, G, d, dv)
+  switch (R) {
+    case 1: RULE(1); break;
+    case 2: RULE(2); break;
+    case 4: RULE(4); break;
+    case 8: RULE(8); break;
+    case 16: RULE(16); break;
+    case 32: RULE(32); break;
+    default: RULE(64); break;
+  }
 #undef RULE
   return vk_check_launch("delta rule");
 }
