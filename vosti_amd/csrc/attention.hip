@@ -903,6 +903,12 @@ __global__ __launch_bounds__(128, 2) void attn_decode_pair_kernel(AttnArgs a) {
 #endif
 #define LOG2E 1.4426950408889634f
 
+// tanh(x) = 1 - 2 / (2^(2 x log2 e) + 1): saturates to +-1 without a branch; its absolute error is a few units of
+// 32-bit rounding at 1, so a capped score is off by that times the cap.
+__device__ __forceinline__ float fast_tanh(float x) {
+  return 1.f - 2.f * __builtin_amdgcn_rcpf(fast_exp2(x * (2.f * LOG2E)) + 1.f);
+}
+
 __device__ __forceinline__ float sink_term(const AttnArgs& a, int head, float M) {
   return fast_exp2(__builtin_fmaf(load_weight(a.sinks, a.sinks_f32, head), LOG2E, -M));
 }
@@ -970,7 +976,7 @@ __device__ __forceinline__ void tile_step_ext(const RowCtx& c, float scale, floa
   if (softcap > 0.f) {
     const float inner = scale / softcap;
 #pragma unroll
-    for (int i = 0; i < S_PER_LANE; ++i) sc[i] = softcap * tanhf(sc[i] * inner);
+    for (int i = 0; i < S_PER_LANE; ++i) sc[i] = softcap * fast_tanh(sc[i] * inner);
   } else {
 #pragma unroll
     for (int i = 0; i < S_PER_LANE; ++i) sc[i] = sc[i] * scale;

@@ -90,15 +90,41 @@ __global__ __launch_bounds__(256) void delta_decay_kernel(float* __restrict__ g,
 }
 
 // The recurrence.  A workgroup of four waves takes 4 * 64 / R value columns of one (sequence, head); a column's state
-// is spread over R neighbouring lanes, lane r of them holding the key channels 16 r .. 16 r + 15 in registers.  The
+// is spread over R neighbouring lanes, lane r of them holding the key channels 8 r .. 8 r + 7 in registers.  The
 // inputs of a chunk of tokens (q, k and the decays of the head, the columns' v, beta) are brought into LDS by the whole
 // workgroup, the next chunk's while this one is computed (global memory -> registers before the chunk's work, registers
 // -> the other LDS buffer after it, one barrier a chunk), so that the walk over the tokens waits for LDS only.  The two
-// sums of a token run over a lane's channels in ascending order and then as a butterfly over the R lanes, whatever the
+// sums of a token run over a lane's channels in ascending order and then as a butterfly over the R lanes (group_sum), whatever the
 // chunks are: a token's arithmetic does not know where a step was cut.  In memory a head's state is [vdim][dim], so
-// that a lane's channels are 64 consecutive bytes and a wave's loads are whole lines.
-#define RULE_DR 16
+// that a lane's channels are 32 consecutive bytes and a wave's loads are whole lines.  The next token's inputs are
+// read from LDS into registers while this token's sums run.
+#define RULE_DR 8
 #define RULE_THREADS 256
+
+// The sum over the R neighbouring lanes of an aligned group, in every lane of the group: a butterfly whose steps stay
+// in the vector unit (quad permutes, the mirrors of a half row and of a row, the swaps of rows and halves), not the
+// shuffle through LDS.  The order of the additions is fixed by R.
+__device__ __forceinline__ float dpp_f(float v, int ctrl_tag) {
+  const int x = __builtin_bit_cast(int, v);
+  int y;
+  switch (ctrl_tag) {
+    case 0: y = __builtin_amdgcn_update_dpp(x, x, 0xB1, 0xF, 0xF, false); break;    // quad_perm [1, 0, 3, 2]
+    case 1: y = __builtin_amdgcn_update_dpp(x, x, 0x4E, 0xF, 0xF, false); break;    // quad_perm [2, 3, 0, 1]
+    case 2: y = __builtin_amdgcn_update_dpp(x, x, 0x141, 0xF, 0xF, false); break;   // row_half_mirror
+    default: y = __builtin_amdgcn_update_dpp(x, x, 0x140, 0xF, 0xF, false); break;  // row_mirror
+  }
+  return __builtin_bit_cast(float, y);
+}
+template <int R>
+__device__ __forceinline__ float group_sum(float v) {
+  if (R >= 2) v = v + dpp_f(v, 0);
+  if (R >= 4) v = v + dpp_f(v, 1);
+  if (R >= 8) v = v + dpp_f(v, 2);
+  if (R >= 16) v = v + dpp_f(v, 3);
+  if (R >= 32) v = v + lane_xor16(v);
+  if (R >= 64) v = v + lane_xor32(v);
+  return v;
+}
 
 template <int R>
 struct RuleShape {
@@ -209,26 +235,38 @@ __global__ __launch_bounds__(RULE_THREADS) void delta_rule_kernel(float* __restr
     const float* base = smem + (chunk & 1) * Sh::BUF;
     if (chunk + 1 < chunks) fetch(chunk + 1);
     const int here = min(TC, n - chunk * TC);
-    for (int tok = 0; tok < here; ++tok) {
+    // The inputs of token `tok` as this lane needs them; asked for one token ahead.
+    float kn[DR], qn[DR], gn[DR], vn, bn;
+    auto read = [&](int tok) {
       const float* kr = base + tok * DMAX + r * DR;
       const float* qr = kr + TC * DMAX;
       const float* gr = qr + TC * DMAX;
-      const float v = base[3 * TC * DMAX + tok * CB + col_in_block];
-      const float beta = base[3 * TC * DMAX + TC * CB + tok];
-      float kk[DR], qq[DR];
-      float dot = 0.f;
 #pragma unroll
       for (int i = 0; i < DR; i += 4) {
         const f32x4 k4 = *reinterpret_cast<const f32x4*>(kr + i), g4 = *reinterpret_cast<const f32x4*>(gr + i);
         const f32x4 q4 = *reinterpret_cast<const f32x4*>(qr + i);
-        kk[i] = k4.x; kk[i + 1] = k4.y; kk[i + 2] = k4.z; kk[i + 3] = k4.w;
-        qq[i] = q4.x; qq[i + 1] = q4.y; qq[i + 2] = q4.z; qq[i + 3] = q4.w;
-        S[i] = S[i] * g4.x; S[i + 1] = S[i + 1] * g4.y; S[i + 2] = S[i + 2] * g4.z; S[i + 3] = S[i + 3] * g4.w;
+        kn[i] = k4.x; kn[i + 1] = k4.y; kn[i + 2] = k4.z; kn[i + 3] = k4.w;
+        qn[i] = q4.x; qn[i + 1] = q4.y; qn[i + 2] = q4.z; qn[i + 3] = q4.w;
+        gn[i] = g4.x; gn[i + 1] = g4.y; gn[i + 2] = g4.z; gn[i + 3] = g4.w;
       }
+      vn = base[3 * TC * DMAX + tok * CB + col_in_block];
+      bn = base[3 * TC * DMAX + TC * CB + tok];
+    };
+    read(0);
+    for (int tok = 0; tok < here; ++tok) {
+      float kk[DR], qq[DR];
+      float dot = 0.f;
+      const float v = vn, beta = bn;
+#pragma unroll
+      for (int i = 0; i < DR; ++i) {
+        kk[i] = kn[i];
+        qq[i] = qn[i];
+        S[i] = S[i] * gn[i];
+      }
+      if (tok + 1 < here) read(tok + 1);
 #pragma unroll
       for (int i = 0; i < DR; ++i) dot = dot + S[i] * kk[i];
-#pragma unroll
-      for (int m = 1; m < R; m <<= 1) dot = dot + __shfl_xor(dot, m, VK_WAVE);
+      dot = group_sum<R>(dot);
       const float u = beta * (v - dot);
       float o = 0.f;
 #pragma unroll
@@ -236,8 +274,7 @@ __global__ __launch_bounds__(RULE_THREADS) void delta_rule_kernel(float* __restr
         S[i] = S[i] + kk[i] * u;
         o = o + S[i] * qq[i];
       }
-#pragma unroll
-      for (int m = 1; m < R; m <<= 1) o = o + __shfl_xor(o, m, VK_WAVE);
+      o = group_sum<R>(o);
       if (col_ok && r == 0) out[((int64_t)(first + chunk * TC + tok) * H + h) * dv + col] = o;
     }
     if (chunk + 1 < chunks) stage((chunk + 1) & 1);
@@ -272,7 +309,7 @@ __global__ __launch_bounds__(64) void delta_out_kernel(elem_t* __restrict__ y, c
 
 extern "C" {
 
-// Lanes that share a value column for key size d: each holds 16 key channels.
+// Lanes that share a value column for key size d: each holds 8 key channels.
 int vk_delta_lanes_per_column(int d) {
   int R = 1;
   while (R < 64 && R * RULE_DR < d) R *= 2;

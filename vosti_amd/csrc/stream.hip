@@ -82,6 +82,86 @@ __global__ __launch_bounds__(STREAM_THREADS) void stream_norm_add_kernel(float* 
   }
 }
 
+// The same two norms for rows of whole 16-byte vectors that fit a workgroup's registers: thread t owns the vectors t,
+// t + 256, ... (NV of them at most), reads them once, and sums their squares element by element in that order.
+template <bool IN_F32, int NV>
+__global__ __launch_bounds__(STREAM_THREADS) void stream_norm_vec_kernel(elem_t* __restrict__ out, const void* __restrict__ x,
+                                                                         const void* __restrict__ w, int w_is_f32, int H, float eps,
+                                                                         float offset) {
+  __shared__ float red[4];
+  const int64_t base = (int64_t)blockIdx.x * H;
+  const int nvec = H / 4;
+  f32x4 v[NV];
+  float part = 0.f;
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const int c = threadIdx.x + j * STREAM_THREADS;
+    v[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (c < nvec) {
+      if (IN_F32) {
+        v[j] = *reinterpret_cast<const f32x4*>(static_cast<const float*>(x) + base + 4 * c);
+      } else {
+        const elem_t* p = static_cast<const elem_t*>(x) + base + 4 * c;
+        v[j] = f32x4{to_f32(p[0]), to_f32(p[1]), to_f32(p[2]), to_f32(p[3])};
+      }
+    }
+    part = part + v[j].x * v[j].x;
+    part = part + v[j].y * v[j].y;
+    part = part + v[j].z * v[j].z;
+    part = part + v[j].w * v[j].w;
+  }
+  const float rr = rsqrtf(stream_block_sum(part, red) / (float)H + eps);
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const int c = threadIdx.x + j * STREAM_THREADS;
+    if (c < nvec) {
+      elem_t* o = out + base + 4 * c;
+      o[0] = from_f32<elem_t>((v[j].x * rr) * (offset + load_weight(w, w_is_f32, 4 * c)));
+      o[1] = from_f32<elem_t>((v[j].y * rr) * (offset + load_weight(w, w_is_f32, 4 * c + 1)));
+      o[2] = from_f32<elem_t>((v[j].z * rr) * (offset + load_weight(w, w_is_f32, 4 * c + 2)));
+      o[3] = from_f32<elem_t>((v[j].w * rr) * (offset + load_weight(w, w_is_f32, 4 * c + 3)));
+    }
+  }
+}
+
+template <int NV>
+__global__ __launch_bounds__(STREAM_THREADS) void stream_norm_add_vec_kernel(float* out, const float* base_rows, const elem_t* __restrict__ y,
+                                                                             const void* __restrict__ w, int w_is_f32, int H, float eps,
+                                                                             float offset, float mult) {
+  __shared__ float red[4];
+  const int64_t base = (int64_t)blockIdx.x * H;
+  const int nvec = H / 4;
+  f32x4 v[NV], b[NV];
+  float part = 0.f;
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const int c = threadIdx.x + j * STREAM_THREADS;
+    v[j] = b[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (c < nvec) {
+      const elem_t* p = y + base + 4 * c;
+      v[j] = f32x4{to_f32(p[0]), to_f32(p[1]), to_f32(p[2]), to_f32(p[3])};
+      b[j] = *reinterpret_cast<const f32x4*>(base_rows + base + 4 * c);
+    }
+    part = part + v[j].x * v[j].x;
+    part = part + v[j].y * v[j].y;
+    part = part + v[j].z * v[j].z;
+    part = part + v[j].w * v[j].w;
+  }
+  const float rr = rsqrtf(stream_block_sum(part, red) / (float)H + eps);
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const int c = threadIdx.x + j * STREAM_THREADS;
+    if (c < nvec) {
+      f32x4 o;
+      o.x = b[j].x + mult * ((v[j].x * rr) * (offset + load_weight(w, w_is_f32, 4 * c)));
+      o.y = b[j].y + mult * ((v[j].y * rr) * (offset + load_weight(w, w_is_f32, 4 * c + 1)));
+      o.z = b[j].z + mult * ((v[j].z * rr) * (offset + load_weight(w, w_is_f32, 4 * c + 2)));
+      o.w = b[j].w + mult * ((v[j].w * rr) * (offset + load_weight(w, w_is_f32, 4 * c + 3)));
+      *reinterpret_cast<f32x4*>(out + base + 4 * c) = o;
+    }
+  }
+}
+
 // out[e] = sum over j < n of coef[j] * states[j * stride + e], added in ascending j from zero.
 __global__ __launch_bounds__(256) void stream_mix_kernel(float* __restrict__ out, const float* __restrict__ states, int64_t stride,
                                                          const void* __restrict__ coef, int coef_is_f32, int n, int64_t numel) {
@@ -120,8 +200,17 @@ int vk_stream_norm(elem_t* out, const void* x, int x_is_f32, const void* w, int 
                    hipStream_t st) {
   VK_REQUIRE(rows >= 0 && H > 0 && eps >= 0.f, "stream norm: bad sizes rows=%d H=%d", rows, H);
   if (rows == 0) return 0;
-  if (x_is_f32) stream_norm_kernel<true><<<rows, STREAM_THREADS, 0, st>>>(out, x, w, w_is_f32, H, eps, offset);
-  else stream_norm_kernel<false><<<rows, STREAM_THREADS, 0, st>>>(out, x, w, w_is_f32, H, eps, offset);
+  const int nv = (H / 4 + STREAM_THREADS - 1) / STREAM_THREADS;
+  if (H % 4 == 0 && nv <= 8 && (uintptr_t)x % 16 == 0) {
+#define NORM_VEC(F32, NV) stream_norm_vec_kernel<F32, NV><<<rows, STREAM_THREADS, 0, st>>>(out, x, w, w_is_f32, H, eps, offset)
+    if (x_is_f32) { if (nv <= 1) NORM_VEC(true, 1); else if (nv <= 2) NORM_VEC(true, 2); else if (nv <= 4) NORM_VEC(true, 4); else NORM_VEC(true, 8); }
+    else { if (nv <= 1) NORM_VEC(false, 1); else if (nv <= 2) NORM_VEC(false, 2); else if (nv <= 4) NORM_VEC(false, 4); else NORM_VEC(false, 8); }
+#undef NORM_VEC
+  } else if (x_is_f32) {
+    stream_norm_kernel<true><<<rows, STREAM_THREADS, 0, st>>>(out, x, w, w_is_f32, H, eps, offset);
+  } else {
+    stream_norm_kernel<false><<<rows, STREAM_THREADS, 0, st>>>(out, x, w, w_is_f32, H, eps, offset);
+  }
   return vk_check_launch("stream norm");
 }
 
@@ -129,7 +218,14 @@ int vk_stream_norm_add(float* out, const float* base, const elem_t* y, const voi
                        float offset, float mult, hipStream_t st) {
   VK_REQUIRE(rows >= 0 && H > 0 && eps >= 0.f, "stream norm-add: bad sizes rows=%d H=%d", rows, H);
   if (rows == 0) return 0;
-  stream_norm_add_kernel<<<rows, STREAM_THREADS, 0, st>>>(out, base, y, w, w_is_f32, H, eps, offset, mult);
+  const int nv = (H / 4 + STREAM_THREADS - 1) / STREAM_THREADS;
+  if (H % 4 == 0 && nv <= 8 && (uintptr_t)out % 16 == 0 && (uintptr_t)base % 16 == 0) {
+#define NORM_ADD_VEC(NV) stream_norm_add_vec_kernel<NV><<<rows, STREAM_THREADS, 0, st>>>(out, base, y, w, w_is_f32, H, eps, offset, mult)
+    if (nv <= 1) NORM_ADD_VEC(1); else if (nv <= 2) NORM_ADD_VEC(2); else if (nv <= 4) NORM_ADD_VEC(4); else NORM_ADD_VEC(8);
+#undef NORM_ADD_VEC
+  } else {
+    stream_norm_add_kernel<<<rows, STREAM_THREADS, 0, st>>>(out, base, y, w, w_is_f32, H, eps, offset, mult);
+  }
   return vk_check_launch("stream norm-add");
 }
 
