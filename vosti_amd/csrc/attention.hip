@@ -349,6 +349,105 @@ __device__ __forceinline__ void init_ctx(RowCtx& c, const AttnArgs& a, int seq, 
   c.scale_log2 = a.scale_log2;
 }
 
+#ifdef VK_BF16
+#define P_PARTS 3
+#else
+#define P_PARTS 1
+#endif
+#define LOG2E 1.4426950408889634f
+
+// tanh(x) = 1 - 2 / (2^(2 x log2 e) + 1): saturates to +-1 without a branch; its absolute error is a few units of
+// 32-bit rounding at 1, so a capped score is off by that times the cap.
+__device__ __forceinline__ float fast_tanh(float x) {
+  return 1.f - 2.f * __builtin_amdgcn_rcpf(fast_exp2(x * (2.f * LOG2E)) + 1.f);
+}
+
+__device__ __forceinline__ float sink_term(const AttnArgs& a, int head, float M) {
+  return fast_exp2(__builtin_fmaf(load_weight(a.sinks, a.sinks_f32, head), LOG2E, -M));
+}
+
+// tile_probs for scores in natural units (already scaled and capped), with kept first keys and unrounded weights.
+__device__ __forceinline__ void tile_probs_ext(float (&sc)[S_PER_LANE], int kb, int g, bool row_ok, int lo, int pos, int keep,
+                                               float& M, float& L, float& ca, frag_t (&pf)[P_PARTS][KEY_SLABS]) {
+  float pr[S_PER_LANE];
+  float psum = 0.f;
+  bool vis[S_PER_LANE];
+  float tmax = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < S_PER_LANE; ++i) {
+    const int key = kb + (i / VK_VEC) * VK_SLAB + g * VK_VEC + (i % VK_VEC);
+    vis[i] = row_ok && key <= pos && (key >= lo || key < keep);
+    tmax = fmaxf(tmax, vis[i] ? sc[i] : -INFINITY);
+  }
+  tmax = fmaxf(tmax, lane_xor16(tmax));
+  tmax = fmaxf(tmax, lane_xor32(tmax));
+  const float m = tmax * LOG2E;             // -inf: the row sees no key of the tile
+  const float Mn = (!(M > -INFINITY) || m > M + MAX_STEP) ? m : M;
+  ca = Mn > -INFINITY ? fast_exp2(M - Mn) : 1.f;
+#pragma unroll
+  for (int i = 0; i < S_PER_LANE; ++i) {
+    pr[i] = vis[i] ? fast_exp2(__builtin_fmaf(sc[i], LOG2E, -Mn)) : 0.f;
+    psum = psum + pr[i];
+  }
+  psum = psum + lane_xor16(psum);
+  psum = psum + lane_xor32(psum);
+  L = __builtin_fmaf(L, ca, psum);
+  M = Mn;
+#pragma unroll
+  for (int ks = 0; ks < KEY_SLABS; ++ks) {
+#ifdef VK_BF16
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      // Each difference is exact: what rounding to 8 bits leaves of a 24-bit number has 16 bits, then 8.
+      const float p = pr[ks * 8 + j];
+      const __bf16 hi = (__bf16)p;
+      const float r1 = p - (float)hi;
+      const __bf16 mid = (__bf16)r1;
+      pf[0][ks][j] = hi;
+      pf[1][ks][j] = mid;
+      pf[2][ks][j] = (__bf16)(r1 - (float)mid);
+    }
+#else
+    pf[0][ks] = f32x4{pr[ks * 4 + 0], pr[ks * 4 + 1], pr[ks * 4 + 2], pr[ks * 4 + 3]};
+#endif
+  }
+}
+
+// The second half of a tile's work for the variant with capped scores: the cap, the probabilities onto the row's state,
+// and P V with the unrounded weights.  vf: the tile's value fragments (from global memory; cleaned here).
+template <int NDT>
+__device__ __forceinline__ void tile_softmax_pv_ext(const RowCtx& c, float scale, float softcap, float (&sc)[S_PER_LANE], int kb,
+                                                    frag_t (&vf)[NDT][KEY_SLABS], float& M, float& L, f32x4 (&ACC)[NDT]) {
+  if (softcap > 0.f) {
+    const float inner = scale / softcap;
+#pragma unroll
+    for (int i = 0; i < S_PER_LANE; ++i) sc[i] = softcap * fast_tanh(sc[i] * inner);
+  } else {
+#pragma unroll
+    for (int i = 0; i < S_PER_LANE; ++i) sc[i] = sc[i] * scale;
+  }
+  frag_t pf[P_PARTS][KEY_SLABS];
+  float ca;
+  const bool fresh = !(M > -INFINITY);
+  tile_probs_ext(sc, kb, c.g, c.row_ok, c.lo, c.pos, c.keep, M, L, ca, pf);
+  scale_state<NDT>(ACC, ca, fresh);
+  if (kb + TILE_KEYS > c.k_len || kb < c.wave_lo) {
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt)
+      if (dt * 16 < c.d) zero_unowned(vf[dt], kb, c.g, c.wave_lo, c.k_len, c.keep);
+  }
+#pragma unroll
+  for (int dt = 0; dt < NDT; ++dt) {
+    if (dt * 16 < c.d) {
+#pragma unroll
+      for (int ks = 0; ks < KEY_SLABS; ++ks) {
+#pragma unroll
+        for (int part = 0; part < P_PARTS; ++part) ACC[dt] = mma_slab(vf[dt][ks], pf[part][ks], ACC[dt]);
+      }
+    }
+  }
+}
+
 // Prompt portions, the kernel for every head size and page size: an item is up
 // to ITEM_ROWS consecutive rows of one sequence, a workgroup takes 16 of them.
 // It has one wave per q head of a kv head (up to 4), so that the waves of a
@@ -448,8 +547,11 @@ __device__ __forceinline__ int key_swz(int row) { return row & 15; }
 __device__ __forceinline__ int val_swz(int row) { return row & 15; }          // rows of 256 bytes
 #endif
 
-template <int DPAD, int NW, int NST = 2>
-__global__ __launch_bounds__(64 * NW, 2) void attn_prefill_lds_kernel(AttnArgs a, int n_items) {
+// EXT: the variant with capped scores, kept first keys, a sink and unrounded weights (see tile_probs_ext): the kept
+// keys' tiles come before the window's, the tiles between are left out, and the three parts of a probability are three
+// products; with EXT unset the code is what it was.
+template <int DPAD, int NW, int NST = 2, bool EXT = false>
+__global__ __launch_bounds__(64 * NW, EXT ? 1 : 2) void attn_prefill_lds_kernel(AttnArgs a, int n_items) {
   constexpr int ROWS_WG = 16 * NW;                       // NW waves, each with one 16-row tile
   constexpr int BPI = ITEM_ROWS / ROWS_WG;               // workgroups per item
   static_assert(ITEM_ROWS % ROWS_WG == 0, "a workgroup's rows must divide an item");
@@ -493,6 +595,13 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_lds_kernel(AttnArgs a
   const int pos_item = k_len - q_len + q_off0;           // position of the item's first row
   const int item_lo = a.window > 0 ? max(0, pos_item - a.window + 1) : 0;
   const int tile_lo = item_lo / TILE_KEYS, tile_hi = (pos_item + rows_item - 1) / TILE_KEYS;
+  // The tiles this workgroup walks: with kept first keys, their tiles (those that lie before the window's) and then the
+  // window's; otherwise tile_lo .. tile_hi.
+  const int keep = EXT && a.window > 0 ? a.keep : 0;
+  const int keep_tiles = (keep + TILE_KEYS - 1) / TILE_KEYS;
+  const int n_before = min(keep_tiles, tile_lo);
+  const int n_tiles = n_before + tile_hi - tile_lo + 1;
+  auto tile_of = [&](int i) { return i < n_before ? i : tile_lo + (i - n_before); };
 
   // ---- this wave's rows ----
   const int rows_wave = min(16, rows_item - 16 * wave);  // <= 0: the wave only helps to load
@@ -544,15 +653,17 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_lds_kernel(AttnArgs a
 #pragma unroll
   for (int dt = 0; dt < NDT; ++dt) ACC[dt] = As[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  issue(tile_lo, 0);
+  issue(tile_of(0), 0);
   // The buffer a tile lies in is a constant in the code of its step (the loop below takes two steps a turn), so that
   // the LDS addresses of the fragments are computed once for the kernel and not added to a buffer's base in every tile.
-  auto step = [&](int t, auto stage_c) {
+  auto step = [&](int i, auto stage_c) {
     constexpr int stage = decltype(stage_c)::value;
+    const int t = tile_of(i);
+    const bool last = i + 1 == n_tiles;
     wait_vm_loads();
     __syncthreads();      // tile t is in LDS; every wave is done with the other buffer
-    if (NST == 2 && t < tile_hi) issue(t + 1, stage ^ 1);
-    if (t * TILE_KEYS + TILE_KEYS > k_len || t * TILE_KEYS < item_lo) {
+    if (NST == 2 && !last) issue(tile_of(i + 1), stage ^ 1);
+    if (t * TILE_KEYS + TILE_KEYS > k_len || (t * TILE_KEYS < item_lo && t * TILE_KEYS + TILE_KEYS > keep)) {
       // Keys outside [item_lo, k_len) may lie in pages this sequence does not own: their values are replaced by
       // zero in LDS, so that stale NaN or Inf cannot reach a sum (their probabilities are zero).  The first and
       // the last tile of an item at most; the same for every wave, which all pass the second barrier.
@@ -560,14 +671,14 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_lds_kernel(AttnArgs a
       unsigned char* vt = lds + stage * STAGE + KT_BYTES;
       for (int e = threadIdx.x; e < DPAD * TILE_KEYS; e += 64 * NW) {
         const int vrow = e / TILE_KEYS, key = e % TILE_KEYS;
-        if (kb + key >= k_len || kb + key < item_lo) {
+        if (kb + key >= k_len || (kb + key < item_lo && kb + key >= keep)) {
           const int col = (key / VK_VEC) ^ val_swz(vrow);
           *reinterpret_cast<elem_t*>(vt + vrow * VRB + col * 16 + (key % VK_VEC) * EB) = (elem_t)0.f;
         }
       }
       __syncthreads();
     }
-    if (t >= wtile_lo && t <= wtile_hi) {
+    if ((t >= wtile_lo || t < keep_tiles) && t <= wtile_hi) {
       const int kb = t * TILE_KEYS;
       const unsigned char* kl = lds + stage * STAGE;
       const unsigned char* vl = kl + KT_BYTES;
@@ -595,10 +706,22 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_lds_kernel(AttnArgs a
       // ---- the row's new maximum, its probabilities, its sums so far under the new maximum ----
       const bool full = rows_wave >= 16 && kb + TILE_KEYS - 1 <= pos_wave &&
                         kb >= (a.window > 0 ? max(0, pos_wave + 15 - a.window + 1) : 0);
-      frag_t pf[KEY_SLABS];
+      frag_t pf[EXT ? P_PARTS : 1][KEY_SLABS];
       float ca;
       const bool fresh = !(Ms > -INFINITY);
-      tile_probs(sc, kb, g, row_ok, lo, pos, a.scale_log2, full, Ms, Ls, ca, pf);
+      if constexpr (EXT) {
+        if (a.softcap > 0.f) {
+          const float inner = a.scale / a.softcap;
+#pragma unroll
+          for (int e = 0; e < S_PER_LANE; ++e) sc[e] = a.softcap * fast_tanh(sc[e] * inner);
+        } else {
+#pragma unroll
+          for (int e = 0; e < S_PER_LANE; ++e) sc[e] = sc[e] * a.scale;
+        }
+        tile_probs_ext(sc, kb, g, row_ok, lo, pos, keep, Ms, Ls, ca, pf);
+      } else {
+        tile_probs(sc, kb, g, row_ok, lo, pos, a.scale_log2, full, Ms, Ls, ca, pf[0]);
+      }
       scale_state<NDT>(As, ca, fresh);
       __builtin_amdgcn_sched_barrier(0);
       // ---- P V onto the segment's sums, column block by column block ----
@@ -612,15 +735,18 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_lds_kernel(AttnArgs a
 #pragma unroll
         for (int ks = 0; ks < KEY_SLABS; ++ks) vf[ks] = *reinterpret_cast<const frag_t*>(vr + (((ks * 4 + g) ^ sw) << 4));
 #pragma unroll
-        for (int ks = 0; ks < KEY_SLABS; ++ks) As[dt] = mma_slab(vf[ks], pf[ks], As[dt]);
+        for (int ks = 0; ks < KEY_SLABS; ++ks) {
+#pragma unroll
+          for (int part = 0; part < (EXT ? P_PARTS : 1); ++part) As[dt] = mma_slab(vf[ks], pf[part][ks], As[dt]);
+        }
       }
       __builtin_amdgcn_s_setprio(0);
     }
-    if (NST == 1 && t < tile_hi) {                         // one buffer: the next tile may come when every wave has read this one
+    if (NST == 1 && !last) {                               // one buffer: the next tile may come when every wave has read this one
       __syncthreads();
-      issue(t + 1, 0);
+      issue(tile_of(i + 1), 0);
     }
-    if ((t + 1) % SEG_TILES == 0 || t == tile_hi) {        // the segment is complete
+    if (last || tile_of(i + 1) / SEG_TILES != t / SEG_TILES) {   // the segment is complete
       fold<NDT>(M, L, ACC, Ms, Ls, As);
       Ms = -INFINITY;
       Ls = 0.f;
@@ -628,11 +754,12 @@ __global__ __launch_bounds__(64 * NW, 2) void attn_prefill_lds_kernel(AttnArgs a
       for (int dt = 0; dt < NDT; ++dt) As[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
     }
   };
-  for (int t = tile_lo; t <= tile_hi; t += 2) {
-    step(t, std::integral_constant<int, 0>{});
-    if (t + 1 <= tile_hi) step(t + 1, std::integral_constant<int, NST == 2 ? 1 : 0>{});
+  for (int i = 0; i < n_tiles; i += 2) {
+    step(i, std::integral_constant<int, 0>{});
+    if (i + 1 < n_tiles) step(i + 1, std::integral_constant<int, NST == 2 ? 1 : 0>{});
   }
   if (row_ok) {
+    if (EXT && a.sinks != nullptr && M > -INFINITY) L = L + sink_term(a, head, M);
     const float inv = L > 0.f ? 1.0f / L : 0.f;
     elem_t* orow = a.out + ((int64_t)tok * a.nq + head) * a.d;
 #pragma unroll
@@ -896,70 +1023,6 @@ __global__ __launch_bounds__(128, 2) void attn_decode_pair_kernel(AttnArgs a) {
 // The reduction order is the one of the kernels above: tiles of 64 keys at absolute positions, four to a segment,
 // segments folded in ascending order; the tiles between the kept keys and the window are left out, which changes
 // no sum.  So the result does not depend on how a sequence was cut into steps.
-#ifdef VK_BF16
-#define P_PARTS 3
-#else
-#define P_PARTS 1
-#endif
-#define LOG2E 1.4426950408889634f
-
-// tanh(x) = 1 - 2 / (2^(2 x log2 e) + 1): saturates to +-1 without a branch; its absolute error is a few units of
-// 32-bit rounding at 1, so a capped score is off by that times the cap.
-__device__ __forceinline__ float fast_tanh(float x) {
-  return 1.f - 2.f * __builtin_amdgcn_rcpf(fast_exp2(x * (2.f * LOG2E)) + 1.f);
-}
-
-__device__ __forceinline__ float sink_term(const AttnArgs& a, int head, float M) {
-  return fast_exp2(__builtin_fmaf(load_weight(a.sinks, a.sinks_f32, head), LOG2E, -M));
-}
-
-// tile_probs for scores in natural units (already scaled and capped), with kept first keys and unrounded weights.
-__device__ __forceinline__ void tile_probs_ext(float (&sc)[S_PER_LANE], int kb, int g, bool row_ok, int lo, int pos, int keep,
-                                               float& M, float& L, float& ca, frag_t (&pf)[P_PARTS][KEY_SLABS]) {
-  float pr[S_PER_LANE];
-  float psum = 0.f;
-  bool vis[S_PER_LANE];
-  float tmax = -INFINITY;
-#pragma unroll
-  for (int i = 0; i < S_PER_LANE; ++i) {
-    const int key = kb + (i / VK_VEC) * VK_SLAB + g * VK_VEC + (i % VK_VEC);
-    vis[i] = row_ok && key <= pos && (key >= lo || key < keep);
-    tmax = fmaxf(tmax, vis[i] ? sc[i] : -INFINITY);
-  }
-  tmax = fmaxf(tmax, lane_xor16(tmax));
-  tmax = fmaxf(tmax, lane_xor32(tmax));
-  const float m = tmax * LOG2E;             // -inf: the row sees no key of the tile
-  const float Mn = (!(M > -INFINITY) || m > M + MAX_STEP) ? m : M;
-  ca = Mn > -INFINITY ? fast_exp2(M - Mn) : 1.f;
-#pragma unroll
-  for (int i = 0; i < S_PER_LANE; ++i) {
-    pr[i] = vis[i] ? fast_exp2(__builtin_fmaf(sc[i], LOG2E, -Mn)) : 0.f;
-    psum = psum + pr[i];
-  }
-  psum = psum + lane_xor16(psum);
-  psum = psum + lane_xor32(psum);
-  L = __builtin_fmaf(L, ca, psum);
-  M = Mn;
-#pragma unroll
-  for (int ks = 0; ks < KEY_SLABS; ++ks) {
-#ifdef VK_BF16
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      // Each difference is exact: what rounding to 8 bits leaves of a 24-bit number has 16 bits, then 8.
-      const float p = pr[ks * 8 + j];
-      const __bf16 hi = (__bf16)p;
-      const float r1 = p - (float)hi;
-      const __bf16 mid = (__bf16)r1;
-      pf[0][ks][j] = hi;
-      pf[1][ks][j] = mid;
-      pf[2][ks][j] = (__bf16)(r1 - (float)mid);
-    }
-#else
-    pf[0][ks] = f32x4{pr[ks * 4 + 0], pr[ks * 4 + 1], pr[ks * 4 + 2], pr[ks * 4 + 3]};
-#endif
-  }
-}
-
 template <int NDT, int NQS, bool V_LATE>
 __device__ __forceinline__ void tile_step_ext(const RowCtx& c, float scale, float softcap, const frag_t (&qf)[NQS], int kb, float& M,
                                               float& L, f32x4 (&ACC)[NDT]) {
@@ -973,34 +1036,7 @@ __device__ __forceinline__ void tile_step_ext(const RowCtx& c, float scale, floa
     __builtin_amdgcn_sched_barrier(0);
     load_values<NDT, false>(c, kb, vf);
   }
-  if (softcap > 0.f) {
-    const float inner = scale / softcap;
-#pragma unroll
-    for (int i = 0; i < S_PER_LANE; ++i) sc[i] = softcap * fast_tanh(sc[i] * inner);
-  } else {
-#pragma unroll
-    for (int i = 0; i < S_PER_LANE; ++i) sc[i] = sc[i] * scale;
-  }
-  frag_t pf[P_PARTS][KEY_SLABS];
-  float ca;
-  const bool fresh = !(M > -INFINITY);
-  tile_probs_ext(sc, kb, c.g, c.row_ok, c.lo, c.pos, c.keep, M, L, ca, pf);
-  scale_state<NDT>(ACC, ca, fresh);
-  if (kb + TILE_KEYS > c.k_len || kb < c.wave_lo) {
-#pragma unroll
-    for (int dt = 0; dt < NDT; ++dt)
-      if (dt * 16 < c.d) zero_unowned(vf[dt], kb, c.g, c.wave_lo, c.k_len, c.keep);
-  }
-#pragma unroll
-  for (int dt = 0; dt < NDT; ++dt) {
-    if (dt * 16 < c.d) {
-#pragma unroll
-      for (int ks = 0; ks < KEY_SLABS; ++ks) {
-#pragma unroll
-        for (int part = 0; part < P_PARTS; ++part) ACC[dt] = mma_slab(vf[dt][ks], pf[part][ks], ACC[dt]);
-      }
-    }
-  }
+  tile_softmax_pv_ext<NDT>(c, scale, softcap, sc, kb, vf, M, L, ACC);
 }
 
 // Prompt rows: attn_prefill_kernel with the four things above.
@@ -1117,6 +1153,84 @@ __global__ __launch_bounds__(64 * PLAIN_WAVES) void attn_decode_ext_kernel(AttnA
 #pragma unroll
     for (int dt = 0; dt < NDT; ++dt)
       if (dt * 16 < a.d) *reinterpret_cast<f32x4*>(&a.part_acc[prow * a.d + dt * 16 + 4 * c.g]) = ACC[dt];
+  }
+}
+
+// Decoded tokens of the same variant where a wave's registers hold two tiles' fragments: attn_decode_seg_kernel's walk
+// (the next tile's keys asked for when this tile's scores are done, its values when this tile's product is), over the
+// tiles of the segment that hold kept first keys or keys of the window.
+template <int DPAD, bool EXACT>
+__global__ __launch_bounds__(64 * SEG_WAVES, 2) void attn_decode_seg_ext_kernel(AttnArgs a) {
+  constexpr int NDT = DPAD / 16, NQS = DPAD / VK_SLAB;
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int G = a.nq / a.nkv, HT = (G + 15) >> 4;
+  const int kvh = blockIdx.y / HT, ht = blockIdx.y - kvh * HT;
+  const int seg = blockIdx.z * SEG_WAVES + wave;
+  const int seq = a.items[2 * blockIdx.x], q_off = a.items[2 * blockIdx.x + 1];
+  const int q_begin = a.cu_q[seq], q_len = a.cu_q[seq + 1] - q_begin;
+  const int k_len = a.k_len[seq];
+  const int tok = q_begin + q_off;
+  const int pos = k_len - q_len + q_off;
+  const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
+  const int keep = a.window > 0 ? a.keep : 0;
+  const int keep_tiles = (keep + TILE_KEYS - 1) / TILE_KEYS, tile_lo = lo / TILE_KEYS;
+  // The segment's tiles that hold visible keys, in ascending order.
+  int tiles[SEG_TILES], nt = 0;
+#pragma unroll
+  for (int j = 0; j < SEG_TILES; ++j) {
+    const int t = seg * SEG_TILES + j;
+    if (t <= pos / TILE_KEYS && (t < keep_tiles || t >= tile_lo)) tiles[nt++] = t;
+  }
+  if (nt == 0) return;   // whole wave; no barrier follows
+
+  RowCtx c;
+  init_ctx(c, a, seq, kvh, k_len);
+  c.r16 = lane & 15;
+  c.g = lane >> 4;
+  c.row_ok = c.r16 < min(16, G - ht * 16);
+  c.pos = pos;
+  c.lo = lo;
+  c.wave_lo = lo;
+  c.keep = keep;
+  const int head = kvh * G + ht * 16 + c.r16;
+  frag_t qf[NQS];
+  load_q<NQS>(a, tok, head, c.row_ok, c.g, qf);
+  frag_t kf[KSUB][NQS];
+  frag_t vf[NDT][KEY_SLABS];
+  load_keys<NQS, EXACT>(c, tiles[0] * TILE_KEYS, kf);
+  load_values<NDT, EXACT>(c, tiles[0] * TILE_KEYS, vf);
+  float M = -INFINITY, L = 0.f;
+  f32x4 ACC[NDT];
+#pragma unroll
+  for (int dt = 0; dt < NDT; ++dt) ACC[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+  for (int j = 0; j < SEG_TILES; ++j) {
+    if (j < nt) {
+      const int kb = tiles[j] * TILE_KEYS;
+      const bool more = j + 1 < nt;
+      const int next = more ? tiles[j + 1 < SEG_TILES ? j + 1 : j] * TILE_KEYS : kb;
+      float sc[S_PER_LANE];
+      tile_scores<NQS, EXACT>(c, kf, qf, sc);
+      __builtin_amdgcn_sched_barrier(0);
+      if (more) load_keys<NQS, EXACT>(c, next, kf);
+      __builtin_amdgcn_sched_barrier(0);
+      tile_softmax_pv_ext<NDT>(c, a.scale, a.softcap, sc, kb, vf, M, L, ACC);
+      __builtin_amdgcn_sched_barrier(0);
+      if (more) load_values<NDT, EXACT>(c, next, vf);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
+  if (!c.row_ok) return;
+  const int64_t prow = ((int64_t)blockIdx.x * a.nq + head) * a.nseg + seg;
+  if (c.g == 0) {
+    a.part_ml[2 * prow] = M;
+    a.part_ml[2 * prow + 1] = L;
+  }
+  if (M > -INFINITY) {
+#pragma unroll
+    for (int dt = 0; dt < NDT; ++dt)
+      if (EXACT || dt * 16 < a.d) *reinterpret_cast<f32x4*>(&a.part_acc[prow * a.d + dt * 16 + 4 * c.g]) = ACC[dt];
   }
 }
 
@@ -1387,6 +1501,28 @@ int vk_paged_attention_capped(elem_t* out, const elem_t* q, const elem_t* kc, co
   a.part_ml = nullptr; a.part_acc = nullptr;
   a.keep = keep; a.scale = scale; a.softcap = softcap; a.sinks = sinks; a.sinks_f32 = sinks_f32;
   const int G = nq / nkv;
+  if (mode == 0 && vk_attn_prefill_shares_tiles(d, P)) {
+    // Key and value tiles through LDS, as for the plain attention; eight waves a workgroup unless they are few.
+    VK_REQUIRE((int64_t)n_items * (ITEM_ROWS / 16) * nq < (1ll << 31), "attention: too many prompt items");
+    const size_t smem = (size_t)4 * TILE_KEYS * d * sizeof(elem_t);
+#define PREFILL_LDS_EXT(DP, NW)                                                                      \
+  do {                                                                                               \
+    static bool raised = false;                                                                      \
+    if (!raised) {                                                                                   \
+      (void)hipFuncSetAttribute((const void*)attn_prefill_lds_kernel<DP, NW, 2, true>,               \
+                                hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);             \
+      raised = true;                                                                                 \
+    }                                                                                                \
+    attn_prefill_lds_kernel<DP, NW, 2, true><<<n_items * (ITEM_ROWS / (16 * NW)) * nq, 64 * NW, smem, st>>>(a, n_items); \
+  } while (0)
+    // (In 32-bit with the widest heads eight waves' registers do not hold the three-part products' operands.)
+    const bool four = 2 * (int64_t)n_items * nq < 3 * (int64_t)attn_device_cus() || (sizeof(elem_t) == 4 && d == 256);
+    if (d == 64) { if (four) PREFILL_LDS_EXT(64, 4); else PREFILL_LDS_EXT(64, 8); }
+    else if (d == 128) { if (four) PREFILL_LDS_EXT(128, 4); else PREFILL_LDS_EXT(128, 8); }
+    else { if (four) PREFILL_LDS_EXT(256, 4); else PREFILL_LDS_EXT(256, 8); }
+#undef PREFILL_LDS_EXT
+    return vk_check_launch("attention (prompt rows, capped scores, shared tiles)");
+  }
   if (mode == 0) {
     const int hpw = G < 4 ? G : 4;
     VK_REQUIRE((int64_t)n_items * (ITEM_ROWS / 16) < (1ll << 31), "attention: too many prompt items");
@@ -1400,8 +1536,25 @@ int vk_paged_attention_capped(elem_t* out, const elem_t* q, const elem_t* kc, co
   VK_REQUIRE(nseg > 0 && nseg <= 65535 && scratch != nullptr, "attention: decode needs nseg in 1..65535 and scratch");
   a.part_ml = scratch;
   a.part_acc = scratch + (((int64_t)n_items * nq * nseg * 2 + 3) & ~(int64_t)3);
+  VK_REQUIRE(nkv * ((G + 15) / 16) <= 65535 && nq <= 65535, "attention: too many heads");
+  if (sizeof(elem_t) * vk_dpad(d) <= 256) {
+    // A wave's registers hold two tiles' fragments: the walk with the next tile in flight.
+    const bool exact = P >= TILE_KEYS && d == vk_dpad(d);
+    const dim3 sgrid(n_items, nkv * ((G + 15) / 16), (nseg + SEG_WAVES - 1) / SEG_WAVES);
+#define DECODE_SEG_EXT(DP)                                                                     \
+  do {                                                                                         \
+    if (exact) attn_decode_seg_ext_kernel<DP, true><<<sgrid, 64 * SEG_WAVES, 0, st>>>(a);      \
+    else attn_decode_seg_ext_kernel<DP, false><<<sgrid, 64 * SEG_WAVES, 0, st>>>(a);           \
+  } while (0)
+    if (d <= 64) DECODE_SEG_EXT(64);
+    else if (d <= 128) DECODE_SEG_EXT(128);
+    else DECODE_SEG_EXT(256);
+#undef DECODE_SEG_EXT
+    if (vk_check_launch("attention (decoded rows, capped scores, wave per segment)")) return 1;
+    attn_combine_kernel<<<dim3(n_items, nq), 64, 0, st>>>(a);
+    return vk_check_launch("attention (combine)");
+  }
   const dim3 grid(n_items, nkv * ((G + 15) / 16), (nseg + PLAIN_WAVES - 1) / PLAIN_WAVES);
-  VK_REQUIRE(grid.y <= 65535 && nq <= 65535, "attention: too many heads");
   const bool late = (int64_t)grid.x * grid.y * nseg > 1024;
 #define DECODE_EXT(DP)                                                                   \
   do {                                                                                   \

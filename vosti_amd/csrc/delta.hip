@@ -90,15 +90,15 @@ __global__ __launch_bounds__(256) void delta_decay_kernel(float* __restrict__ g,
 }
 
 // The recurrence.  A workgroup of four waves takes 4 * 64 / R value columns of one (sequence, head); a column's state
-// is spread over R neighbouring lanes, lane r of them holding the key channels 8 r .. 8 r + 7 in registers.  The
+// is spread over R neighbouring lanes, lane r of them holding DR consecutive key channels in registers (4 for key sizes up to 256: more lanes
+// a column mean more waves and shorter sums a token).  The
 // inputs of a chunk of tokens (q, k and the decays of the head, the columns' v, beta) are brought into LDS by the whole
 // workgroup, the next chunk's while this one is computed (global memory -> registers before the chunk's work, registers
 // -> the other LDS buffer after it, one barrier a chunk), so that the walk over the tokens waits for LDS only.  The two
 // sums of a token run over a lane's channels in ascending order and then as a butterfly over the R lanes (group_sum), whatever the
 // chunks are: a token's arithmetic does not know where a step was cut.  In memory a head's state is [vdim][dim], so
-// that a lane's channels are 32 consecutive bytes and a wave's loads are whole lines.  The next token's inputs are
+// that a lane's channels are consecutive and a wave's loads are whole lines.  The next token's inputs are
 // read from LDS into registers while this token's sums run.
-#define RULE_DR 8
 #define RULE_THREADS 256
 
 // The sum over the R neighbouring lanes of an aligned group, in every lane of the group: a butterfly whose steps stay
@@ -126,9 +126,9 @@ __device__ __forceinline__ float group_sum(float v) {
   return v;
 }
 
-template <int R>
+template <int R, int DR>
 struct RuleShape {
-  static constexpr int DMAX = RULE_DR * R;                       // key channels this instance holds
+  static constexpr int DMAX = DR * R;                            // key channels this instance holds
   static constexpr int TC = 2048 / DMAX < 16 ? 2048 / DMAX : 16; // tokens a chunk
   static constexpr int CB = 4 * 64 / R;                          // value columns a workgroup
   static constexpr int BUF = (TC * (3 * DMAX + CB + 1) + 3) / 4 * 4;   // floats of one LDS buffer: k, q, g, v, beta
@@ -136,14 +136,14 @@ struct RuleShape {
   static constexpr int NV = (TC * CB + RULE_THREADS - 1) / RULE_THREADS;
 };
 
-template <int R>
+template <int R, int DR>
 __global__ __launch_bounds__(RULE_THREADS) void delta_rule_kernel(float* __restrict__ out, const float* __restrict__ qkv, int64_t ld, int q_col,
                                                                   int k_col, int v_col, const float* __restrict__ decay,
                                                                   const elem_t* __restrict__ b, int64_t ldb, float* state, int64_t state_stride,
                                                                   const int32_t* __restrict__ cu_q, const int32_t* __restrict__ positions,
                                                                   const int32_t* __restrict__ slots, int H, int G, int d, int dv) {
-  using Sh = RuleShape<R>;
-  constexpr int DR = RULE_DR, DMAX = Sh::DMAX, TC = Sh::TC, CB = Sh::CB;
+  using Sh = RuleShape<R, DR>;
+  constexpr int DMAX = Sh::DMAX, TC = Sh::TC, CB = Sh::CB;
   __shared__ __attribute__((aligned(16))) float smem[2 * Sh::BUF];
   const int s = blockIdx.x, h = blockIdx.y;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -309,10 +309,11 @@ __global__ __launch_bounds__(64) void delta_out_kernel(elem_t* __restrict__ y, c
 
 extern "C" {
 
-// Lanes that share a value column for key size d: each holds 8 key channels.
+// Key channels a lane holds, and lanes that share a value column, for key size d.
+static int rule_channels_per_lane(int d) { return d <= 256 ? 4 : (d <= 512 ? 8 : 16); }
 int vk_delta_lanes_per_column(int d) {
   int R = 1;
-  while (R < 64 && R * RULE_DR < d) R *= 2;
+  while (R < 64 && R * rule_channels_per_lane(d) < d) R *= 2;
   return R;
 }
 
@@ -357,23 +358,29 @@ int vk_delta_rule(float* out, const float* qkv, int64_t ld, int q_col, int k_col
                   float* state, int64_t state_stride, const int32_t* cu_q, const int32_t* positions, const int32_t* slots, int S, int H, int G,
                   int d, int dv, hipStream_t st) {
   VK_REQUIRE(S >= 0 && H > 0 && G > 0 && H % G == 0 && d > 0 && dv > 0, "delta rule: bad sizes H=%d G=%d d=%d dv=%d", H, G, d, dv);
-  VK_REQUIRE(d <= 64 * RULE_DR, "delta rule: key size %d exceeds %d", d, 64 * RULE_DR);
+  VK_REQUIRE(d <= 1024, "delta rule: key size %d exceeds 1024", d);
   VK_REQUIRE(state_stride >= (int64_t)H * d * dv, "delta rule: the state is too small");
   if (S == 0) return 0;
-  const int R = vk_delta_lanes_per_column(d);
+  const int R = vk_delta_lanes_per_column(d), DR = rule_channels_per_lane(d);
   const int cols = 4 * 64 / R;
   const dim3 grid(S, H, (dv + cols - 1) / cols);
   VK_REQUIRE(grid.y <= 65535 && grid.z <= 65535, "delta rule: too many heads or columns");
-#define RULE(RR) \
-  delta_rule_kernel<RR><<<grid, RULE_THREADS, 0, st>>>(out, qkv, ld, q_col, k_col, v_col, decay, b, ldb, state, state_stride, cu_q, positions, slots, H, G, d, dv)
-  switch (R) {
-    case 1: RULE(1); break;
-    case 2: RULE(2); break;
-    case 4: RULE(4); break;
-    case 8: RULE(8); break;
-    case 16: RULE(16); break;
-    case 32: RULE(32); break;
-    default: RULE(64); break;
+#define RULE(RR, DD) \
+  delta_rule_kernel<RR, DD><<<grid, RULE_THREADS, 0, st>>>(out, qkv, ld, q_col, k_col, v_col, decay, b, ldb, state, state_stride, cu_q, positions, slots, H, G, d, dv)
+  if (DR == 4) {
+    switch (R) {
+      case 1: RULE(1, 4); break;
+      case 2: RULE(2, 4); break;
+      case 4: RULE(4, 4); break;
+      case 8: RULE(8, 4); break;
+      case 16: RULE(16, 4); break;
+      case 32: RULE(32, 4); break;
+      default: RULE(64, 4); break;
+    }
+  } else if (DR == 8) {
+    RULE(64, 8);
+  } else {
+    RULE(64, 16);
   }
 #undef RULE
   return vk_check_launch("delta rule");
