@@ -68,6 +68,7 @@ ALONE = {
     "delta": config([delta_layer(2, 1, 16, 8, conv=3)], width=32, vocab=50),
     "delta_one_tap": config([delta_layer(2, 2, 24, 24, conv=1)], width=32, vocab=50),
     "feed_forward": config([delta_layer(1, 1, 8, 8, conv=2, ff=56)], width=32, vocab=50, residual_mult=1.3),
+    "sizes_that_need_padding": config([delta_layer(3, 1, 10, 5, conv=3, ff=20), attention_layer(3, 3, 6, 10, size=8, keep_first=1, ff=12)], width=24, vocab=33),
     "shared_keys": config([attention_layer(2, 1, 16, 32, size=9, keep_first=1), attention_layer(2, 1, 16, 32, size=9, keep_first=1, kv_from=0)],
                           width=32, vocab=50),
 }
@@ -117,6 +118,26 @@ def test_whole_prompt_portions_and_decoding_agree(models, name, dtype):
     for what, cuts in cuttings.items():
         got = run_cut(eng, 1, tokens, cuts)
         assert deviation(got, whole) < SAME[dtype], what
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("head", [64, 128, 256])
+def test_head_sizes_and_pages_of_the_kernels_that_share_tiles(tmp_path, head, dtype):
+    """Head sizes 64, 128 and 256 with pages of 64: prompt rows go through the kernel that passes key tiles through LDS,
+    decoded rows through the one that keeps the next tile in flight; windows and kept keys that end inside tiles,
+    several prompt items, a prompt after cached keys."""
+    cfg = config([attention_layer(4, 2, head, head, size=150, keep_first=70, softcap=15.0, ff=64),
+                  attention_layer(4, 2, head, head, size=150, keep_first=70, softcap=15.0, kv_from=0)], width=64, vocab=90)
+    w = random_weights(cfg, 31)
+    folder = write_model(tmp_path / f"h{head}", cfg, w)
+    n = 420
+    tokens = tokens_for(cfg, n, 14)
+    want = plain_logits(cfg, w, tokens)
+    eng = engine(folder, dtype, num_pages=16, page_size=64)
+    whole = run_cut(eng, 0, tokens, [n])
+    assert deviation(whole, want) < TOLERANCE[dtype]
+    for cuts in ([200, 150, 70], [n - 30] + [1] * 30, [64, 64, 129, 100, 63]):
+        assert deviation(run_cut(eng, 1, tokens, cuts), whole) < SAME[dtype], cuts
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

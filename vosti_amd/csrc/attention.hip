@@ -436,6 +436,8 @@ __device__ __forceinline__ void tile_softmax_pv_ext(const RowCtx& c, float scale
     for (int dt = 0; dt < NDT; ++dt)
       if (dt * 16 < c.d) zero_unowned(vf[dt], kb, c.g, c.wave_lo, c.k_len, c.keep);
   }
+  // A sum takes its products in the order (key slab, part).  (Walking several column blocks side by side, so that no MFMA
+  // follows one it depends on, costs the decode kernels more registers than a wave has: they spill.)
 #pragma unroll
   for (int dt = 0; dt < NDT; ++dt) {
     if (dt * 16 < c.d) {
@@ -726,18 +728,40 @@ __global__ __launch_bounds__(64 * NW, EXT ? 1 : 2) void attn_prefill_lds_kernel(
       __builtin_amdgcn_sched_barrier(0);
       // ---- P V onto the segment's sums, column block by column block ----
       __builtin_amdgcn_s_setprio(1);
+      if constexpr (EXT) {
+        // Four column blocks at a time, so that the three parts' products of one sum do not follow each other.
+        constexpr int DG = NDT < 4 ? NDT : 4;
 #pragma unroll
-      for (int dt = 0; dt < NDT; ++dt) {
-        const int vrow = dt * 16 + r16;
-        const unsigned char* vr = vl + vrow * VRB;
-        const int sw = val_swz(vrow);
-        frag_t vf[KEY_SLABS];
+        for (int dt0 = 0; dt0 < NDT; dt0 += DG) {
+          frag_t vf[DG][KEY_SLABS];
 #pragma unroll
-        for (int ks = 0; ks < KEY_SLABS; ++ks) vf[ks] = *reinterpret_cast<const frag_t*>(vr + (((ks * 4 + g) ^ sw) << 4));
+          for (int j = 0; j < DG; ++j) {
+            const int vrow = (dt0 + j) * 16 + r16;
+            const unsigned char* vr = vl + vrow * VRB;
+            const int sw = val_swz(vrow);
 #pragma unroll
-        for (int ks = 0; ks < KEY_SLABS; ++ks) {
+            for (int ks = 0; ks < KEY_SLABS; ++ks) vf[j][ks] = *reinterpret_cast<const frag_t*>(vr + (((ks * 4 + g) ^ sw) << 4));
+          }
 #pragma unroll
-          for (int part = 0; part < (EXT ? P_PARTS : 1); ++part) As[dt] = mma_slab(vf[ks], pf[part][ks], As[dt]);
+          for (int ks = 0; ks < KEY_SLABS; ++ks) {
+#pragma unroll
+            for (int part = 0; part < P_PARTS; ++part) {
+#pragma unroll
+              for (int j = 0; j < DG; ++j) As[dt0 + j] = mma_slab(vf[j][ks], pf[part][ks], As[dt0 + j]);
+            }
+          }
+        }
+      } else {
+#pragma unroll
+        for (int dt = 0; dt < NDT; ++dt) {
+          const int vrow = dt * 16 + r16;
+          const unsigned char* vr = vl + vrow * VRB;
+          const int sw = val_swz(vrow);
+          frag_t vf[KEY_SLABS];
+#pragma unroll
+          for (int ks = 0; ks < KEY_SLABS; ++ks) vf[ks] = *reinterpret_cast<const frag_t*>(vr + (((ks * 4 + g) ^ sw) << 4));
+#pragma unroll
+          for (int ks = 0; ks < KEY_SLABS; ++ks) As[dt] = mma_slab(vf[ks], pf[0][ks], As[dt]);
         }
       }
       __builtin_amdgcn_s_setprio(0);
@@ -1175,14 +1199,15 @@ __global__ __launch_bounds__(64 * SEG_WAVES, 2) void attn_decode_seg_ext_kernel(
   const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
   const int keep = a.window > 0 ? a.keep : 0;
   const int keep_tiles = (keep + TILE_KEYS - 1) / TILE_KEYS, tile_lo = lo / TILE_KEYS;
-  // The segment's tiles that hold visible keys, in ascending order.
-  int tiles[SEG_TILES], nt = 0;
+  // The segment's tiles that hold visible keys, as a mask of SEG_TILES bits.
+  unsigned wanted = 0;
 #pragma unroll
   for (int j = 0; j < SEG_TILES; ++j) {
     const int t = seg * SEG_TILES + j;
-    if (t <= pos / TILE_KEYS && (t < keep_tiles || t >= tile_lo)) tiles[nt++] = t;
+    if (t <= pos / TILE_KEYS && (t < keep_tiles || t >= tile_lo)) wanted |= 1u << j;
   }
-  if (nt == 0) return;   // whole wave; no barrier follows
+  wanted = __builtin_amdgcn_readfirstlane(wanted);
+  if (wanted == 0) return;   // whole wave; no barrier follows
 
   RowCtx c;
   init_ctx(c, a, seq, kvh, k_len);
@@ -1198,18 +1223,20 @@ __global__ __launch_bounds__(64 * SEG_WAVES, 2) void attn_decode_seg_ext_kernel(
   load_q<NQS>(a, tok, head, c.row_ok, c.g, qf);
   frag_t kf[KSUB][NQS];
   frag_t vf[NDT][KEY_SLABS];
-  load_keys<NQS, EXACT>(c, tiles[0] * TILE_KEYS, kf);
-  load_values<NDT, EXACT>(c, tiles[0] * TILE_KEYS, vf);
+  const int first_kb = (seg * SEG_TILES + __builtin_ctz(wanted)) * TILE_KEYS;
+  load_keys<NQS, EXACT>(c, first_kb, kf);
+  load_values<NDT, EXACT>(c, first_kb, vf);
   float M = -INFINITY, L = 0.f;
   f32x4 ACC[NDT];
 #pragma unroll
   for (int dt = 0; dt < NDT; ++dt) ACC[dt] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
   for (int j = 0; j < SEG_TILES; ++j) {
-    if (j < nt) {
-      const int kb = tiles[j] * TILE_KEYS;
-      const bool more = j + 1 < nt;
-      const int next = more ? tiles[j + 1 < SEG_TILES ? j + 1 : j] * TILE_KEYS : kb;
+    if ((wanted >> j) & 1u) {
+      const int kb = (seg * SEG_TILES + j) * TILE_KEYS;
+      const unsigned rest = j + 1 < SEG_TILES ? wanted >> (j + 1) : 0u;
+      const bool more = rest != 0;
+      const int next = more ? kb + (1 + __builtin_ctz(rest)) * TILE_KEYS : kb;
       float sc[S_PER_LANE];
       tile_scores<NQS, EXACT>(c, kf, qf, sc);
       __builtin_amdgcn_sched_barrier(0);

@@ -293,9 +293,11 @@ __global__ __launch_bounds__(RULE_THREADS) void delta_rule_kernel(float* __restr
   }
 }
 
-// y[t, h, :] = o / sqrt(mean(o^2) + eps) * w * sigmoid(gate[t, h, :]), stored as elements.  One wave per (token, head).
-__global__ __launch_bounds__(64) void delta_out_kernel(elem_t* __restrict__ y, const float* __restrict__ o, const elem_t* __restrict__ gate,
-                                                       int64_t ldg, const void* __restrict__ w, int w_is_f32, int H, int dv, float eps) {
+// y[t, h, :] = o / sqrt(mean(o^2) + eps) * w * sigmoid(gate[t, h, :]), stored as elements in rows of length ldy; the
+// columns beyond the heads are set to zero (a projection with padded columns reads them).  One wave per (token, head).
+__global__ __launch_bounds__(64) void delta_out_kernel(elem_t* __restrict__ y, int64_t ldy, const float* __restrict__ o,
+                                                       const elem_t* __restrict__ gate, int64_t ldg, const void* __restrict__ w, int w_is_f32,
+                                                       int H, int dv, float eps) {
   const int t = blockIdx.x / H, h = blockIdx.x - t * H;
   const float* row = o + ((int64_t)t * H + h) * dv;
   float part = 0.f;
@@ -303,8 +305,10 @@ __global__ __launch_bounds__(64) void delta_out_kernel(elem_t* __restrict__ y, c
   const float rr = rsqrtf(wave_sum_xor(part) / (float)dv + eps);
   for (int c = threadIdx.x; c < dv; c += 64) {
     const float gt = sigmoid_f(to_f32(gate[(int64_t)t * ldg + (int64_t)h * dv + c]));
-    y[((int64_t)t * H + h) * dv + c] = from_f32<elem_t>(((row[c] * rr) * load_weight(w, w_is_f32, c)) * gt);
+    y[(int64_t)t * ldy + (int64_t)h * dv + c] = from_f32<elem_t>(((row[c] * rr) * load_weight(w, w_is_f32, c)) * gt);
   }
+  if (h == H - 1)
+    for (int64_t c = (int64_t)H * dv + threadIdx.x; c < ldy; c += 64) y[(int64_t)t * ldy + c] = from_f32<elem_t>(0.f);
 }
 
 extern "C" {
@@ -386,12 +390,12 @@ int vk_delta_rule(float* out, const float* qkv, int64_t ld, int q_col, int k_col
   return vk_check_launch("delta rule");
 }
 
-int vk_delta_out(elem_t* y, const float* o, const elem_t* gate, int64_t ldg, const void* w, int w_is_f32, int T, int H, int dv, float eps,
-                 hipStream_t st) {
-  VK_REQUIRE(T >= 0 && H > 0 && dv > 0 && ldg >= (int64_t)H * dv, "delta read-out: bad sizes");
+int vk_delta_out(elem_t* y, int64_t ldy, const float* o, const elem_t* gate, int64_t ldg, const void* w, int w_is_f32, int T, int H, int dv,
+                 float eps, hipStream_t st) {
+  VK_REQUIRE(T >= 0 && H > 0 && dv > 0 && ldg >= (int64_t)H * dv && ldy >= (int64_t)H * dv, "delta read-out: bad sizes");
   if (T == 0) return 0;
   VK_REQUIRE((int64_t)T * H < (1ll << 31), "delta read-out: too many rows");
-  delta_out_kernel<<<T * H, 64, 0, st>>>(y, o, gate, ldg, w, w_is_f32, H, dv, eps);
+  delta_out_kernel<<<T * H, 64, 0, st>>>(y, ldy, o, gate, ldg, w, w_is_f32, H, dv, eps);
   return vk_check_launch("delta read-out");
 }
 

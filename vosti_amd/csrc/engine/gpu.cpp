@@ -111,7 +111,7 @@ struct Kernels::Fn {
   int (*delta_unit)(P, int64_t, int, int, int, int, float, float, hipStream_t);
   int (*delta_decay)(P, CP, CP, CP, int, int, int, int, hipStream_t);
   int (*delta_rule)(P, CP, int64_t, int, int, int, CP, CP, int64_t, P, int64_t, CP, CP, CP, int, int, int, int, int, hipStream_t);
-  int (*delta_out)(P, CP, CP, int64_t, CP, int, int, int, int, float, hipStream_t);
+  int (*delta_out)(P, int64_t, CP, CP, int64_t, CP, int, int, int, int, float, hipStream_t);
 };
 
 static constexpr int KERNEL_ABI = 14;
@@ -579,14 +579,15 @@ Tensor Kernels::delta_rule(const Tensor& qkv, int q_col, int k_col, int v_col, c
   return out;
 }
 
-Tensor Kernels::delta_out(const Tensor& o, const Tensor& gate, const Tensor& w, int H, int dv, float eps) {
+Tensor Kernels::delta_out(const Tensor& o, const Tensor& gate, const Tensor& w, int H, int dv, float eps, int64_t width) {
   expect(o, "delta read-out", DType::F32);
   expect(gate, "gate", dtype_);
   if (o.shape.size() != 3 || o.dim(1) != H || o.dim(2) != dv || gate.shape.size() != 2 || gate.dim(0) != o.dim(0) || gate.dim(1) != (int64_t)H * dv)
     throw EngineError("delta read-out: " + o.describe() + " with gate " + gate.describe());
   const int wf = norm_weight(w, "read-out norm weight", dv);
-  Tensor y = empty({o.dim(0), (int64_t)H * dv});
-  call(fn_->delta_out(y.data, o.data, gate.data, gate.dim(1), w.data, wf, (int)o.dim(0), H, dv, eps, stream));
+  if (width < (int64_t)H * dv) throw EngineError("delta read-out: a row of " + std::to_string(width) + " does not hold the heads");
+  Tensor y = empty({o.dim(0), width});
+  call(fn_->delta_out(y.data, width, o.data, gate.data, gate.dim(1), w.data, wf, (int)o.dim(0), H, dv, eps, stream));
   return y;
 }
 

@@ -162,7 +162,8 @@ class Kernels {
   Tensor delta_decay(const Tensor& a, const Tensor& dt_bias, const Tensor& A_log, int H, int d);
   Tensor delta_rule(const Tensor& qkv, int q_col, int k_col, int v_col, const Tensor& decay, const Tensor& b, int64_t b_col, Tensor& state,
                     const Tensor& cu_q, const Tensor& positions, const Tensor& slots, int H, int G, int d, int dv);
-  Tensor delta_out(const Tensor& o, const Tensor& gate, const Tensor& w, int H, int dv, float eps);
+  // width: the row length of the result (at least H * dv; the columns beyond are zero).
+  Tensor delta_out(const Tensor& o, const Tensor& gate, const Tensor& w, int H, int dv, float eps, int64_t width);
   int segment_keys() const { return segment_keys_; }
   int item_rows() const { return item_rows_; }
 

@@ -559,11 +559,16 @@ class SwiGLU : public FeedForward {
     return {{"gate_proj.weight", {inter_, hidden_}}, {"up_proj.weight", {inter_, hidden_}}, {"down_proj.weight", {hidden_, inter_}}};
   }
   void load(std::map<std::string, Tensor>& t) override {
-    w_gate_up_ = stack_rows({need(t, "gate_proj.weight"), need(t, "up_proj.weight")});
-    w_down_ = need(t, "down_proj.weight");
+    // An intermediate size that is no multiple of 8 is padded with zero rows (and zero columns of the down projection):
+    // the products' reduction axis must be whole 16-byte vectors, and silu(0) * 0 adds nothing.
+    const int64_t padded = round_up(inter_, 8);
+    w_gate_up_ = stack_rows({pad_matrix(need(t, "gate_proj.weight"), padded, hidden_), pad_matrix(need(t, "up_proj.weight"), padded, hidden_)});
+    w_down_ = pad_matrix(need(t, "down_proj.weight"), hidden_, padded);
+    inter_run_ = padded;
   }
   int64_t gemm_floats(int64_t T) const {
-    return std::max(kernels.gemm_workspace_floats(T, 2 * inter_, hidden_, true), kernels.gemm_workspace_floats(T, hidden_, inter_));
+    const int64_t inter = inter_run_ ? inter_run_ : inter_;
+    return std::max(kernels.gemm_workspace_floats(T, 2 * inter, hidden_, true), kernels.gemm_workspace_floats(T, hidden_, inter));
   }
   int64_t workspace_floats(HostStep& step) override {
     int64_t T = 0;
@@ -578,7 +583,7 @@ class SwiGLU : public FeedForward {
   }
 
  private:
-  int64_t hidden_, inter_;
+  int64_t hidden_, inter_, inter_run_ = 0;   // inter_run_: the intermediate size as the kernels see it
   Tensor w_gate_up_, w_down_;
 };
 
@@ -701,7 +706,7 @@ class ChannelDelta : public Mixer {
     A_log_ = need(t, "A_log");
     dt_bias_ = need(t, "dt_bias");
     out_norm_ = need(t, "out_norm.weight");
-    w_o_ = need(t, "o_proj.weight");
+    w_o_ = pad_matrix(need(t, "o_proj.weight"), hidden_, v_);      // the read-out's width as whole 16-byte vectors
   }
   CacheNeed cache_need() const override {
     CacheNeed n;
@@ -731,7 +736,7 @@ class ChannelDelta : public Mixer {
     const Tensor decay = k.delta_decay(a, dt_bias_, A_log_, H_, d_);
     const Tensor o = k.delta_rule(qkv, 0, (int)qk_, (int)(2 * qk_), decay, proj, beta_col_, cache.state, ctx.cu_q, ctx.positions, ctx.state_slots,
                                   H_, G_, d_, dv_);
-    return k.gemm(k.delta_out(o, gate, out_norm_, H_, dv_, eps_), w_o_);
+    return k.gemm(k.delta_out(o, gate, out_norm_, H_, dv_, eps_, v_), w_o_);
   }
 
  private:

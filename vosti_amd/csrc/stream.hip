@@ -172,6 +172,23 @@ __global__ __launch_bounds__(256) void stream_mix_kernel(float* __restrict__ out
   out[e] = acc;
 }
 
+// The same, four consecutive elements a thread (numel and stride multiples of 4, 16-byte aligned).
+__global__ __launch_bounds__(256) void stream_mix_vec_kernel(f32x4* __restrict__ out, const f32x4* __restrict__ states, int64_t stride4,
+                                                             const void* __restrict__ coef, int coef_is_f32, int n, int64_t numel4) {
+  const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= numel4) return;
+  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+  for (int j = 0; j < n; ++j) {
+    const float cj = load_weight(coef, coef_is_f32, j);
+    const f32x4 v = states[j * stride4 + e];
+    acc.x = acc.x + cj * v.x;
+    acc.y = acc.y + cj * v.y;
+    acc.z = acc.z + cj * v.z;
+    acc.w = acc.w + cj * v.w;
+  }
+  out[e] = acc;
+}
+
 __global__ __launch_bounds__(256) void gather_rows_f32_kernel(float* __restrict__ out, const float* __restrict__ x,
                                                               const int32_t* __restrict__ rows, int H) {
   const float* src = x + (int64_t)rows[blockIdx.x] * H;
@@ -233,7 +250,11 @@ int vk_stream_mix(float* out, const float* states, int64_t stride, const void* c
                   hipStream_t st) {
   VK_REQUIRE(n > 0 && numel >= 0 && stride >= numel, "stream mix: bad sizes n=%d numel=%lld stride=%lld", n, (long long)numel, (long long)stride);
   if (numel == 0) return 0;
-  stream_mix_kernel<<<(unsigned)((numel + 255) / 256), 256, 0, st>>>(out, states, stride, coef, coef_is_f32, n, numel);
+  if (numel % 4 == 0 && stride % 4 == 0 && (uintptr_t)out % 16 == 0 && (uintptr_t)states % 16 == 0)
+    stream_mix_vec_kernel<<<(unsigned)((numel / 4 + 255) / 256), 256, 0, st>>>(reinterpret_cast<f32x4*>(out), reinterpret_cast<const f32x4*>(states),
+                                                                              stride / 4, coef, coef_is_f32, n, numel / 4);
+  else
+    stream_mix_kernel<<<(unsigned)((numel + 255) / 256), 256, 0, st>>>(out, states, stride, coef, coef_is_f32, n, numel);
   return vk_check_launch("stream mix");
 }
 
