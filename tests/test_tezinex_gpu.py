@@ -69,6 +69,8 @@ ALONE = {
     "delta_one_tap": config([delta_layer(2, 2, 24, 24, conv=1)], width=32, vocab=50),
     "feed_forward": config([delta_layer(1, 1, 8, 8, conv=2, ff=56)], width=32, vocab=50, residual_mult=1.3),
     "sizes_that_need_padding": config([delta_layer(3, 1, 10, 5, conv=3, ff=20), attention_layer(3, 3, 6, 10, size=8, keep_first=1, ff=12)], width=24, vocab=33),
+    "shared_keys_seen_further_back": config([attention_layer(2, 2, 16, 16, size=5, keep_first=0), delta_layer(1, 1, 8, 8, conv=2),
+                                             attention_layer(2, 2, 16, 16, size=23, keep_first=4, kv_from=0)], width=32, vocab=50),
     "shared_keys": config([attention_layer(2, 1, 16, 32, size=9, keep_first=1), attention_layer(2, 1, 16, 32, size=9, keep_first=1, kv_from=0)],
                           width=32, vocab=50),
 }
@@ -81,8 +83,10 @@ def test_each_mechanism_alone(tmp_path, name, dtype):
     w = random_weights(cfg, 3, decay_rank=3, gate_rank=9)
     folder = write_model(tmp_path / name, cfg, w)
     tokens = tokens_for(cfg, 45, 1)
-    got = run_cut(engine(folder, dtype), 0, tokens, [45])
-    assert deviation(got, plain_logits(cfg, w, tokens)) < TOLERANCE[dtype]
+    want = plain_logits(cfg, w, tokens)
+    eng = engine(folder, dtype)
+    assert deviation(run_cut(eng, 0, tokens, [45]), want) < TOLERANCE[dtype]
+    assert deviation(run_cut(eng, 1, tokens, [9, 2, 17] + [1] * 17), want) < TOLERANCE[dtype]
 
 
 def test_the_residual_stream_and_the_depth_average_are_32_bit(tmp_path):

@@ -312,6 +312,19 @@ bool DecoderModel::replayable() {
 std::vector<CacheNeed> DecoderModel::cache_needs() {
   std::vector<CacheNeed> out;
   for (const ScheduleEntry& e : spec_.schedule) out.push_back(e.cache_from >= 0 ? CacheNeed{} : layers_[e.layer]->mixer().cache_need());
+  // An execution that reads another's pages may look further back than their owner does: the pages are kept for the
+  // widest window and the most kept first keys of all who read them (a reader of all keys keeps all).
+  for (size_t i = 0; i < spec_.schedule.size(); ++i) {
+    const int from = spec_.schedule[i].cache_from;
+    if (from < 0) continue;
+    const CacheNeed reader = layers_[spec_.schedule[i].layer]->mixer().cache_need();
+    CacheNeed& owner = out[from];
+    if (reader.kind != CacheNeed::Pages || owner.kind != CacheNeed::Pages) continue;      // the pool reports what does not fit
+    if (reader.num_kv_heads != owner.num_kv_heads || reader.head_dim != owner.head_dim)
+      throw ConfigError("schedule entry " + std::to_string(i) + " reads the cache of entry " + std::to_string(from) + ", whose heads are of another number or size");
+    owner.window = (owner.window == 0 || reader.window == 0) ? 0 : std::max(owner.window, reader.window);
+    owner.keep_first = owner.window == 0 ? 0 : std::max(owner.keep_first, reader.keep_first);
+  }
   return out;
 }
 
