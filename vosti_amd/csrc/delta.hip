@@ -89,6 +89,32 @@ __global__ __launch_bounds__(256) void delta_decay_kernel(float* __restrict__ g,
   g[e] = expf(-expf(load_weight(A_log, w_is_f32, col / d)) * sp);
 }
 
+// The two unit norms and the decays of a token in one launch: workgroup (token, j) is q's head j, k's head j - G, or
+// the decays of head j - 2 G; the arithmetic is delta_unit_kernel's and delta_decay_kernel's.
+__global__ __launch_bounds__(64) void delta_prep_kernel(float* x, int64_t ld, int q_col, int k_col, int G, int H, int d, float unit_eps,
+                                                        float q_scale, float* __restrict__ g, const elem_t* __restrict__ a,
+                                                        const void* __restrict__ dt_bias, const void* __restrict__ A_log, int w_is_f32) {
+  const int per = 2 * G + H;
+  const int t = blockIdx.x / per, j = blockIdx.x - t * per;
+  if (j < 2 * G) {
+    const bool is_q = j < G;
+    float* row = x + (int64_t)t * ld + (is_q ? q_col + (int64_t)j * d : k_col + (int64_t)(j - G) * d);
+    float part = 0.f;
+    for (int c = threadIdx.x; c < d; c += 64) part = part + row[c] * row[c];
+    const float r = (is_q ? q_scale : 1.f) / sqrtf(wave_sum_xor(part) + unit_eps);
+    for (int c = threadIdx.x; c < d; c += 64) row[c] = row[c] * r;
+  } else {
+    const int h = j - 2 * G;
+    const float rate = expf(load_weight(A_log, w_is_f32, h));
+    for (int c = threadIdx.x; c < d; c += 64) {
+      const int64_t e = ((int64_t)t * H + h) * d + c;
+      const float z = to_f32(a[e]) + load_weight(dt_bias, w_is_f32, h * d + c);
+      const float sp = z > 20.f ? z : log1pf(expf(z));
+      g[e] = expf(-rate * sp);
+    }
+  }
+}
+
 // The recurrence.  A workgroup of four waves takes 4 * 64 / R value columns of one (sequence, head); a column's state
 // is spread over R neighbouring lanes, lane r of them holding DR consecutive key channels in registers (4 for key sizes up to 256: more lanes
 // a column mean more waves and shorter sums a token).  The
@@ -264,15 +290,16 @@ __global__ __launch_bounds__(RULE_THREADS) void delta_rule_kernel(float* __restr
         S[i] = S[i] * gn[i];
       }
       if (tok + 1 < here) read(tok + 1);
+      // Fused multiply-adds, written out: one instruction and one rounding a step.
 #pragma unroll
-      for (int i = 0; i < DR; ++i) dot = dot + S[i] * kk[i];
+      for (int i = 0; i < DR; ++i) dot = __builtin_fmaf(S[i], kk[i], dot);
       dot = group_sum<R>(dot);
       const float u = beta * (v - dot);
       float o = 0.f;
 #pragma unroll
       for (int i = 0; i < DR; ++i) {
-        S[i] = S[i] + kk[i] * u;
-        o = o + S[i] * qq[i];
+        S[i] = __builtin_fmaf(kk[i], u, S[i]);
+        o = __builtin_fmaf(S[i], qq[i], o);
       }
       o = group_sum<R>(o);
       if (col_ok && r == 0) out[((int64_t)(first + chunk * TC + tok) * H + h) * dv + col] = o;
@@ -353,6 +380,16 @@ int vk_delta_decay(float* g, const elem_t* a, const void* dt_bias, const void* A
   if (numel == 0) return 0;
   delta_decay_kernel<<<(unsigned)((numel + 255) / 256), 256, 0, st>>>(g, a, dt_bias, A_log, w_is_f32, d, H * d, numel);
   return vk_check_launch("decay");
+}
+
+// x[:, q_col ..] (G heads of d) and x[:, k_col ..] become unit vectors (q times q_scale); g [T, H, d] = the decays of a [T, H d].
+int vk_delta_prep(float* x, int64_t ld, int q_col, int k_col, int T, int G, int H, int d, float unit_eps, float q_scale, float* g,
+                  const elem_t* a, const void* dt_bias, const void* A_log, int w_is_f32, hipStream_t st) {
+  VK_REQUIRE(T >= 0 && G > 0 && H > 0 && d > 0 && ld >= (int64_t)G * d + (q_col > k_col ? q_col : k_col), "delta prep: bad sizes");
+  if (T == 0) return 0;
+  VK_REQUIRE((int64_t)T * (2 * G + H) < (1ll << 31), "delta prep: too many rows");
+  delta_prep_kernel<<<T * (2 * G + H), 64, 0, st>>>(x, ld, q_col, k_col, G, H, d, unit_eps, q_scale, g, a, dt_bias, A_log, w_is_f32);
+  return vk_check_launch("delta prep");
 }
 
 // out [T, H, dv] floats.  qkv: float rows of length ld with q (G heads of d) at q_col, k at k_col, v (H heads of dv) at

@@ -110,11 +110,12 @@ struct Kernels::Fn {
   int (*delta_conv)(P, CP, int64_t, CP, P, int64_t, int64_t, CP, CP, CP, CP, int, int, int, int, hipStream_t);
   int (*delta_unit)(P, int64_t, int, int, int, int, float, float, hipStream_t);
   int (*delta_decay)(P, CP, CP, CP, int, int, int, int, hipStream_t);
+  int (*delta_prep)(P, int64_t, int, int, int, int, int, int, float, float, P, CP, CP, CP, int, hipStream_t);
   int (*delta_rule)(P, CP, int64_t, int, int, int, CP, CP, int64_t, P, int64_t, CP, CP, CP, int, int, int, int, int, hipStream_t);
   int (*delta_out)(P, int64_t, CP, CP, int64_t, CP, int, int, int, int, float, hipStream_t);
 };
 
-static constexpr int KERNEL_ABI = 14;
+static constexpr int KERNEL_ABI = 15;
 
 Kernels::Kernels(const std::string& lib_dir, const std::string& name) : name_(name), fn_(new Fn) {
   if (name == "bf16") dtype_ = DType::BF16;
@@ -143,7 +144,7 @@ Kernels::Kernels(const std::string& lib_dir, const std::string& name) : name_(na
   VK(embed_sinusoid, "vk_embed_sinusoid"); VK(stream_norm, "vk_stream_norm"); VK(stream_norm_add, "vk_stream_norm_add");
   VK(stream_mix, "vk_stream_mix"); VK(gather_rows_f32, "vk_gather_rows_f32"); VK(softcap, "vk_softcap");
   VK(qkv_post_bias, "vk_qkv_post_bias"); VK(paged_attention_capped, "vk_paged_attention_capped");
-  VK(delta_conv, "vk_delta_conv"); VK(delta_unit, "vk_delta_unit"); VK(delta_decay, "vk_delta_decay"); VK(delta_rule, "vk_delta_rule");
+  VK(delta_conv, "vk_delta_conv"); VK(delta_prep, "vk_delta_prep"); VK(delta_unit, "vk_delta_unit"); VK(delta_decay, "vk_delta_decay"); VK(delta_rule, "vk_delta_rule");
   VK(delta_out, "vk_delta_out");
 #undef VK
   segment_keys_ = fn_->attn_segment_keys();
@@ -556,6 +557,21 @@ Tensor Kernels::delta_decay(const Tensor& a, const Tensor& dt_bias, const Tensor
   if (norm_weight(A_log, "A_log", H) != wf) throw EngineError("decay: dt_bias and A_log must have one type");
   Tensor g = empty({a.dim(0), H, d}, DType::F32);
   call(fn_->delta_decay(g.data, a.data, dt_bias.data, A_log.data, wf, (int)a.dim(0), H, d, stream));
+  return g;
+}
+
+Tensor Kernels::delta_prep(Tensor& x, int64_t q_col, int64_t k_col, int G, int H, int d, float unit_eps, float q_scale, const Tensor& a,
+                           const Tensor& dt_bias, const Tensor& A_log) {
+  expect(x, "delta rule input", DType::F32);
+  expect(a, "decay input", dtype_);
+  if (x.shape.size() != 2 || a.shape.size() != 2 || a.dim(0) != x.dim(0) || a.dim(1) != (int64_t)H * d ||
+      std::max(q_col, k_col) + (int64_t)G * d > x.dim(1) || q_col < 0 || k_col < 0)
+    throw EngineError("delta prep: input " + x.describe() + ", decay input " + a.describe());
+  const int wf = norm_weight(dt_bias, "dt_bias", (int64_t)H * d);
+  if (norm_weight(A_log, "A_log", H) != wf) throw EngineError("decay: dt_bias and A_log must have one type");
+  Tensor g = empty({a.dim(0), H, d}, DType::F32);
+  call(fn_->delta_prep(x.data, x.dim(1), (int)q_col, (int)k_col, (int)x.dim(0), G, H, d, unit_eps, q_scale, g.data, a.data, dt_bias.data,
+                       A_log.data, wf, stream));
   return g;
 }
 

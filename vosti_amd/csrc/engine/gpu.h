@@ -160,6 +160,9 @@ class Kernels {
                     const Tensor& positions, const Tensor& slots);
   void delta_unit(Tensor& x, int64_t col0, int heads, int d, float eps, float scale);
   Tensor delta_decay(const Tensor& a, const Tensor& dt_bias, const Tensor& A_log, int H, int d);
+  // Both unit norms (q at q_col times q_scale, k at k_col; G heads of d each) and the decays, in one launch; returns the decays.
+  Tensor delta_prep(Tensor& x, int64_t q_col, int64_t k_col, int G, int H, int d, float unit_eps, float q_scale, const Tensor& a,
+                    const Tensor& dt_bias, const Tensor& A_log);
   Tensor delta_rule(const Tensor& qkv, int q_col, int k_col, int v_col, const Tensor& decay, const Tensor& b, int64_t b_col, Tensor& state,
                     const Tensor& cu_q, const Tensor& positions, const Tensor& slots, int H, int G, int d, int dv);
   // width: the row length of the result (at least H * dv; the columns beyond are zero).

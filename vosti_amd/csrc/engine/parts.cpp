@@ -731,9 +731,7 @@ class ChannelDelta : public Mixer {
     const Tensor a = k.gemm_columns(proj, decay_col_, w_decay_up_);
     const Tensor gate = k.gemm_columns(proj, gate_col_, w_gate_up_);
     Tensor qkv = k.delta_conv(proj, conv_, cache.state, state_floats(), ctx.inputs.at("delta.token_seq"), ctx.cu_q, ctx.positions, ctx.state_slots);
-    k.delta_unit(qkv, 0, G_, d_, unit_eps_, 1.f / std::sqrt((float)d_));
-    k.delta_unit(qkv, qk_, G_, d_, unit_eps_, 1.f);
-    const Tensor decay = k.delta_decay(a, dt_bias_, A_log_, H_, d_);
+    const Tensor decay = k.delta_prep(qkv, 0, qk_, G_, H_, d_, unit_eps_, 1.f / std::sqrt((float)d_), a, dt_bias_, A_log_);
     const Tensor o = k.delta_rule(qkv, 0, (int)qk_, (int)(2 * qk_), decay, proj, beta_col_, cache.state, ctx.cu_q, ctx.positions, ctx.state_slots,
                                   H_, G_, d_, dv_);
     return k.gemm(k.delta_out(o, gate, out_norm_, H_, dv_, eps_, v_), w_o_);
