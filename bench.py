@@ -517,7 +517,7 @@ def tezinex_config(width, heads, kv_heads, ff, layers, vocab):
     a layer's matrix work is that of a Qwen3 layer of the same sizes."""
     def attention(kv_from=None):
         m = {"dim": 128, "vdim": 128, "heads": heads, "kv_heads": kv_heads, "mask": {"size": 1024, "keep_first": 16},
-             "scale": 128 ** -0.5, "softcap": 30.0}
+             "scale": 128 ** -0.5, "softcap": 20.0}
         if kv_from is not None:
             m["kv_from"] = kv_from
         return {"type": "attention", "mixer": m, "mlp": {"kind": "dense", "ff": ff}}
@@ -527,7 +527,7 @@ def tezinex_config(width, heads, kv_heads, ff, layers, vocab):
     for i in range(layers):
         kind = i % 4
         out.append(delta if kind in (0, 3) else attention(i - 1 if kind == 2 else None))
-    return {"architecture": "Tezinex", "layers": out, "logit_softcap": 30.0, "norm": {"eps": 1e-6}, "residual_mult": 0.7, "vocab": vocab,
+    return {"architecture": "Tezinex", "layers": out, "logit_softcap": 20.0, "norm": {"eps": 1e-5}, "residual_mult": 0.5, "vocab": vocab,
             "width": width}
 
 

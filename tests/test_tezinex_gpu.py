@@ -204,7 +204,7 @@ def marked_attention_model(size, keep_first):
     tokens differ.  So whether that one key is visible moves the logits by far more than any tolerance."""
     W, d, vocab = 32, 16, 30
     cfg = config([attention_layer(1, 1, d, d, size=size, keep_first=keep_first, scale=0.25, softcap=50.0)], width=W, vocab=vocab,
-                 residual_mult=6.0, logit_softcap=30.0)
+                 residual_mult=6.0, logit_softcap=28.0)
     w = {n: t.float() for n, t in random_weights(cfg, 11).items()}
     g = torch.Generator().manual_seed(4)
     half, extra = W // 2, W - 1

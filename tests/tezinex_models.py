@@ -39,7 +39,7 @@ MIXED = config([
 ], width=64, vocab=97)
 # Delta layers only; wide key size (several lanes a column), one head.
 DELTAS = config([delta_layer(1, 1, 96, 48, conv=3), delta_layer(2, 1, 8, 72, conv=4, ff=40)], width=48, vocab=61, residual_mult=1.0,
-                logit_softcap=30.0)
+                logit_softcap=26.0)
 # One attention layer alone, all q heads on one kv head, the head size of the kernels' widest tiles.
 ATTENTION = config([attention_layer(4, 1, 128, 128, size=40, keep_first=3, ff=None)], width=96, vocab=130, residual_mult=0.9)
 
