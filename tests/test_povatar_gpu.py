@@ -1,0 +1,314 @@
+"""The Povatar decoder through the native engine against the plain implementation (tests/plain_povatar.py).
+
+Every test builds its own small model.  The engine is driven through its step function (given tokens in, logits out:
+what bin/trace_run drives) and through its scheduler (``generate``).  In float32 the engine must agree with the plain
+float64 implementation to a few units of 32-bit rounding; in bfloat16 to what rounding the matrix products to 16 bits
+costs.  Two cuttings of the same tokens through the engine must agree far closer than either does with the plain
+implementation: nothing may depend on portions, batches, pages or slots."""
+import copy
+
+import numpy as np
+import pytest
+import torch
+
+import plain_povatar as plain
+from povatar_models import CONFIGS, MIXED, STRETCH, config, layer, left, moe, random_weights, right, write_model
+
+pytestmark = pytest.mark.gpu
+
+TOLERANCE = {"float32": 2e-4, "bfloat16": 6e-2}      # of the logits' root mean square
+SAME = {"float32": 2e-5, "bfloat16": 2e-5}           # two cuttings of the same tokens through the engine
+
+
+@pytest.fixture(scope="module")
+def models(tmp_path_factory):
+    out = {}
+    for seed, (name, cfg) in enumerate(CONFIGS.items()):
+        w = random_weights(cfg, 20 + seed)
+        out[name] = (write_model(tmp_path_factory.mktemp(name), cfg, w), cfg, w)
+    return out
+
+
+def engine(folder, dtype, num_pages=24, page_size=16, max_num_seqs=4, **kw):
+    from vosti_amd.engine.native import NativeEngine
+    return NativeEngine(folder, dtype=dtype, num_pages=num_pages, page_size=page_size, max_num_seqs=max_num_seqs,
+                        enable_prefix_cache=False, graphs=kw.pop("graphs", False), **kw)
+
+
+def tokens_for(cfg, n, seed):
+    return torch.randint(0, cfg["vocab"], (n,), generator=torch.Generator().manual_seed(seed)).tolist()
+
+
+def run_cut(eng, rid, tokens, cuts, finish=True):
+    """All logits of one request fed in portions of the given sizes."""
+    rows, at = [], 0
+    for c in cuts:
+        rows.append(eng.trace_step([(rid, tokens[at:at + c], list(range(c)))]))
+        at += c
+    assert at == len(tokens)
+    if finish:
+        eng.trace_finish(rid)
+    return np.concatenate(rows, 0)
+
+
+def deviation(got, want):
+    """Largest row deviation as a fraction of the logits' root mean square."""
+    want = np.asarray(want, dtype=np.float64)
+    return float(np.sqrt(((got - want) ** 2).mean(-1)).max() / np.sqrt((want ** 2).mean()))
+
+
+def plain_logits(cfg, w, tokens):
+    return plain.forward(cfg, w, tokens, torch.float64).numpy()
+
+
+# ------------------------------------------------------------------------------------------ each mechanism alone
+NO_LEFT = left(1, 1, 8, 8, size=4, rot_dims=2)            # a small half beside the one under test
+NO_RIGHT = right(1, 4, 4, 1, 1, conv=1)
+ALONE = {
+    "attention": config([layer(left(4, 2, 16, 16, size=12, rot_dims=8, scaling=STRETCH), NO_RIGHT, None)], width=32, vocab=50),
+    "attention_unstretched_whole_head_rotation": config([layer(left(2, 1, 32, 32, size=9, rot_dims=32, base=77.0), NO_RIGHT, None)], width=32, vocab=50),
+    "attention_wide_values_one_block": config([layer(left(2, 2, 8, 48, size=500, rot_dims=4), NO_RIGHT, None)], width=32, vocab=50),
+    "attention_blocks_of_one": config([layer(left(2, 1, 16, 16, size=1, rot_dims=16, scale=1.0), NO_RIGHT, None)], width=32, vocab=50),
+    "state_space": config([layer(NO_LEFT, right(4, 8, 16, 2, 2, conv=3), None)], width=32, vocab=50),
+    "state_space_one_tap_one_group": config([layer(NO_LEFT, right(3, 24, 24, 1, 1, conv=1), None)], width=32, vocab=50),
+    "state_space_wide_state": config([layer(NO_LEFT, right(2, 40, 100, 2, 5, conv=5), None)], width=32, vocab=50),
+    "experts": config([layer(NO_LEFT, NO_RIGHT, moe(7, 2, 20))], width=32, vocab=50, embed_scale=1.0),
+    "experts_all_chosen": config([layer(NO_LEFT, NO_RIGHT, moe(4, 4, 56))], width=32, vocab=50),
+    "experts_many_of_one": config([layer(NO_LEFT, NO_RIGHT, moe(70, 1, 8))], width=32, vocab=50),
+}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", sorted(ALONE))
+def test_each_mechanism_alone(tmp_path, name, dtype):
+    cfg = ALONE[name]
+    w = random_weights(cfg, 3)
+    folder = write_model(tmp_path / name, cfg, w)
+    tokens = tokens_for(cfg, 45, 1)
+    want = plain_logits(cfg, w, tokens)
+    eng = engine(folder, dtype)
+    assert deviation(run_cut(eng, 0, tokens, [45]), want) < TOLERANCE[dtype]
+    assert deviation(run_cut(eng, 1, tokens, [9, 2, 17] + [1] * 17), want) < TOLERANCE[dtype]
+
+
+def test_the_residual_stream_is_32_bit(tmp_path):
+    """Many layers with small updates on a large embedding: a stream rounded to 16 bits between layers would lose them."""
+    cfg = config([layer(NO_LEFT, NO_RIGHT, None) for _ in range(12)], width=32, vocab=40, embed_scale=40.0)
+    w = random_weights(cfg, 5)
+    for n in w:
+        if n.endswith(".out"):
+            w[n] = (w[n].float() * 0.05).to(torch.bfloat16)
+    w["embed"] = (w["embed"].float() * 40.0).to(torch.bfloat16)
+    folder = write_model(tmp_path / "deep", cfg, w)
+    tokens = tokens_for(cfg, 20, 2)
+    got = run_cut(engine(folder, "bfloat16"), 0, tokens, [20])
+    assert deviation(got, plain_logits(cfg, w, tokens)) < 1.5e-2
+
+
+# ----------------------------------------------------------------------------- cuttings, batches, pages and slots
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", sorted(CONFIGS))
+def test_whole_prompt_portions_and_decoding_agree(models, name, dtype):
+    folder, cfg, w = models[name]
+    n = 150
+    tokens = tokens_for(cfg, n, 7)
+    want = plain_logits(cfg, w, tokens)
+    eng = engine(folder, dtype, page_size=16 if name == "MIXED" else 64)
+    whole = run_cut(eng, 0, tokens, [n])
+    assert deviation(whole, want) < TOLERANCE[dtype]
+    # The first tokens of a sequence on their own rows.
+    assert deviation(whole[:4], want[:4]) < TOLERANCE[dtype]
+    cuttings = {
+        "token by token": [1] * n,
+        "portions down to two tokens": [2, 3, 16, 2, 1, 31, 2, 33, 5, 1, 1, 2, 17, 32, 2],
+        "a prompt and then decoding": [n - 60] + [1] * 60,
+        "portions that end on page borders": [16, 48, 64, 22],
+    }
+    for what, cuts in cuttings.items():
+        got = run_cut(eng, 1, tokens, cuts)
+        assert deviation(got, whole) < SAME[dtype], what
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_unequal_requests_in_one_batch(models, dtype):
+    """Portions of some requests beside single tokens of others, a request left out of a step, against each alone."""
+    folder, cfg, w = models["MIXED"]
+    lengths = [70, 23, 41, 5]
+    seqs = [tokens_for(cfg, n, 30 + i) for i, n in enumerate(lengths)]
+    eng = engine(folder, dtype)
+    alone = [run_cut(eng, 10 + i, s, [len(s)]) for i, s in enumerate(seqs)]
+    at = [0] * 4
+    got = [[] for _ in seqs]
+    step = 0
+    while any(a < n for a, n in zip(at, lengths)):
+        entries, who = [], []
+        for i, s in enumerate(seqs):
+            if at[i] >= lengths[i] or (step + i) % 5 == 4:        # finished, or left out of this step
+                continue
+            c = min([7, 1, 2, 1][(step + i) % 4], lengths[i] - at[i])
+            entries.append((i, s[at[i]:at[i] + c], list(range(c))))
+            who.append((i, c))
+            at[i] += c
+        step += 1
+        if not entries:
+            continue
+        rows = eng.trace_step(entries)
+        r = 0
+        for i, c in who:
+            got[i].append(rows[r:r + c])
+            r += c
+    for i in range(4):
+        assert deviation(np.concatenate(got[i], 0), alone[i]) < SAME[dtype], i
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_pages_and_slots_are_used_again(models, dtype):
+    """A pool of one request's pages and one state slot: every request starts in what the one before left."""
+    folder, cfg, w = models["MIXED"]
+    eng = engine(folder, dtype, num_pages=4, page_size=16, max_num_seqs=1)
+    for i, n in enumerate([60, 17, 64, 33]):
+        tokens = tokens_for(cfg, n, 50 + i)
+        got = run_cut(eng, i, tokens, [n // 2, n - n // 2 - 3, 1, 1, 1])
+        assert deviation(got, plain_logits(cfg, w, tokens)) < TOLERANCE[dtype], i
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_long_decoding_past_many_blocks(models, dtype):
+    folder, cfg, w = models["MIXED"]
+    n = 300
+    tokens = tokens_for(cfg, n, 9)
+    eng = engine(folder, dtype, num_pages=20)
+    got = run_cut(eng, 0, tokens, [40] + [1] * (n - 40))
+    assert deviation(got, plain_logits(cfg, w, tokens)) < TOLERANCE[dtype]
+
+
+# ------------------------------------------------------------------------------- a key that stands out, at every edge
+def marked_attention_model(size, head=16, page=16):
+    """One layer whose attention has one head whose query and key are constant directions, so that every query scores
+    `big` on a key wherever that key's token is the mark (token 1) and about zero elsewhere, and whose value carries the
+    mark into the logits: the logits move if and only if the marked key is visible."""
+    cfg = config([layer(left(1, 1, head, head, size=size, rot_dims=2, base=1e6, scale=1.0), NO_RIGHT, None)], width=32, vocab=12, embed_scale=1.0)
+    w = random_weights(cfg, 77)
+    W = cfg["width"]
+    embed = torch.zeros(12, W)
+    embed[:, 0] = 1.0                      # every token: a constant channel that makes the query
+    embed[1, 1] = 6.0                      # the mark: a channel that makes the key and the value
+    embed[2:, 2:] = torch.randn(10, W - 2, generator=torch.Generator().manual_seed(3)) * 0.2
+    w["embed"] = embed.to(torch.bfloat16)
+    q = torch.zeros(head, W)
+    k = torch.zeros(head, W)
+    v = torch.zeros(head, W)
+    q[head - 1, 0] = 8.0                   # the last dimension of the head is not rotated
+    k[head - 1, 1] = 4.0
+    v[:, 1] = 1.0
+    w["l0.norm1"] = torch.ones(W).to(torch.bfloat16)
+    w["l0.mix.left.q"], w["l0.mix.left.k"], w["l0.mix.left.v"] = q.to(torch.bfloat16), k.to(torch.bfloat16), v.to(torch.bfloat16)
+    return cfg, w
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_marked_key_is_seen_exactly_inside_its_block(tmp_path, dtype):
+    size, page = 24, 16
+    cfg, w = marked_attention_model(size)
+    folder = write_model(tmp_path / "marked", cfg, w)
+    eng = engine(folder, dtype, num_pages=16, page_size=page)
+    n = 100
+    rid = 0
+    # (marked position, asking position): first and last of a block, across a block's border, at page borders, far away.
+    cases = [(24, 24), (24, 47), (24, 48), (23, 24), (47, 47), (47, 48), (0, 23), (0, 24), (31, 32), (32, 47), (48, 71), (48, 72),
+             (5, 95), (72, 95), (71, 95), (95, 95), (96, 99), (95, 96)]
+    for mark, ask in cases:
+        tokens = [2 + (i * 7) % 10 for i in range(n)]
+        base = list(tokens)
+        tokens[mark] = 1
+        visible = mark <= ask and mark // size == ask // size
+        p_marked = plain_logits(cfg, w, tokens)[ask]
+        p_base = plain_logits(cfg, w, base)[ask]
+        moved = np.abs(p_marked - p_base).max()
+        if mark != ask:
+            assert (moved > 0.05) == visible, (mark, ask, moved)        # the plain implementation itself, first
+        for cuts in ([n], [ask] + [1] * (n - ask) if ask else [n], [mark + 1, n - mark - 1] if mark + 1 < n else [n], [3, 2] + [5] * 19):
+            got = run_cut(eng, rid, tokens, cuts)[ask]
+            rid += 1
+            assert np.sqrt(((got - p_marked) ** 2).mean()) < TOLERANCE[dtype] * np.sqrt((p_marked ** 2).mean()) + 1e-3, (mark, ask, cuts[:3])
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_the_constant_in_the_denominator(tmp_path, dtype):
+    """Scores far below zero: without the 1 in the denominator the weights would still sum to 1 and the output would be a
+    mean of values; with it the output all but vanishes."""
+    cfg, w = marked_attention_model(50)
+    w["l0.mix.left.q"] = (-w["l0.mix.left.q"].float()).to(torch.bfloat16)
+    folder = write_model(tmp_path / "sink", cfg, w)
+    tokens = [1] * 30
+    want = plain_logits(cfg, w, tokens)
+    got = run_cut(engine(folder, dtype), 0, tokens, [30])
+    assert deviation(got, want) < TOLERANCE[dtype]
+    # The plain implementation itself: the same scores through an ordinary softmax give another answer.
+    h = plain.weighted_norm(plain.embed(tokens, w["embed"], 1.0, torch.float64), w["l0.norm1"].double(), cfg["norm"]["eps"])
+    out = plain.block_attention(h, w, "l0.mix.left.", cfg["layers"][0]["mixer"]["left"])
+    assert out.abs().max() < 1e-6
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_the_recurrence_cut_between_any_two_tokens(tmp_path, dtype):
+    cfg = config([layer(NO_LEFT, right(2, 16, 16, 1, 2, conv=4), None), layer(NO_LEFT, right(4, 8, 8, 2, 1, conv=2), moe(4, 2, 16))], width=32, vocab=50)
+    w = random_weights(cfg, 8)
+    folder = write_model(tmp_path / "cuts", cfg, w)
+    n = 40
+    tokens = tokens_for(cfg, n, 4)
+    eng = engine(folder, dtype)
+    whole = run_cut(eng, 0, tokens, [n])
+    assert deviation(whole, plain_logits(cfg, w, tokens)) < TOLERANCE[dtype]
+    for cut in range(1, n):
+        assert deviation(run_cut(eng, cut, tokens, [cut, n - cut]), whole) < SAME[dtype], cut
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_slow_decay_remembers_the_first_token(tmp_path, dtype):
+    """A head that decays slowly keeps the first token's input for hundreds of tokens: a state that is lost or reset on the
+    way shows in the last logits."""
+    cfg = config([layer(NO_LEFT, right(1, 8, 8, 1, 1, conv=2), None)], width=32, vocab=20)
+    w = random_weights(cfg, 12)
+    w["l0.mix.right.A_log"] = torch.full((1,), -9.0).to(torch.bfloat16)
+    w["l0.mix.right.dt_bias"] = torch.full((1,), 1.0).to(torch.bfloat16)
+    w["l0.mix.right.D"] = torch.zeros(1).to(torch.bfloat16)
+    folder = write_model(tmp_path / "slow", cfg, w)
+    n = 260
+    a = tokens_for(cfg, n, 5)
+    b = list(a)
+    b[0] = (a[0] + 1) % cfg["vocab"]
+    want_a, want_b = plain_logits(cfg, w, a), plain_logits(cfg, w, b)
+    assert np.abs(want_a[-1] - want_b[-1]).max() > 0.02          # the plain implementation: the first token still matters
+    eng = engine(folder, dtype, num_pages=20)
+    for tokens, want in ((a, want_a), (b, want_b)):
+        assert deviation(run_cut(eng, 0, tokens, [100, 7] + [1] * (n - 107)), want) < TOLERANCE[dtype]
+
+
+# ------------------------------------------------------------------------------------------------- generation
+@pytest.mark.parametrize("graphs", [False, True])
+def test_greedy_generation_through_the_scheduler(models, graphs):
+    """create_engine -> the scheduler, the step function, the sampler: the tokens are the plain implementation's."""
+    from vosti_amd.engine import create_engine
+    from vosti_amd.sampling.params import SamplingParams
+    folder, cfg, w = models["MIXED"]
+    prompts = [tokens_for(cfg, n, 60 + i) for i, n in enumerate([19, 3, 40])]
+    eng = create_engine(folder, dtype="float32", num_pages=24, page_size=16, max_num_seqs=4, graphs=graphs)
+    out = eng.generate(prompts, SamplingParams(max_tokens=12, ignore_eos=True))
+    for prompt, got in zip(prompts, out):
+        seq = list(prompt)
+        for _ in range(12):
+            seq.append(int(plain.forward(cfg, w, seq)[-1].argmax()))
+        assert list(got) == seq[len(prompt):]
+
+
+def test_configuration_errors(tmp_path):
+    from vosti_amd.config.registry import describe
+    bad = copy.deepcopy(MIXED)
+    bad["layers"][0]["type"] = "serial"
+    with pytest.raises(Exception, match="unknown mixer type"):
+        describe(bad)
+    bad = copy.deepcopy(MIXED)
+    bad["layers"][0]["mlp"]["router"]["top"] = 9
+    with pytest.raises(Exception, match="top"):
+        describe(bad)

@@ -72,7 +72,15 @@ struct AttnArgs {
   float scale = 0.f, softcap = 0.f;   // score = softcap * tanh(q.k * scale / softcap); softcap 0: score = q.k * scale
   const void* sinks = nullptr;        // [nq] or null: exp(sinks[head]) joins the softmax's denominator, with no value
   int sinks_f32 = 0;
+  int block = 0;          // > 0 (without a window): positions are cut into blocks of this size, and a row sees the keys of its own block only
 };
+
+// The first key that the row at position `pos` sees.  It never decreases with pos, so the smallest row of a wave or an
+// item bounds them all.
+__device__ __forceinline__ int first_visible(const AttnArgs& a, int pos) {
+  if (a.block > 0) return pos - pos % a.block;
+  return a.window > 0 ? max(0, pos - a.window + 1) : 0;
+}
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
@@ -480,8 +488,8 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(AttnArgs a, int heads
   const int tok = q_begin + q_off + c.r16;
   const int pos0 = k_len - q_len + q_off;
   c.pos = pos0 + c.r16;
-  c.lo = a.window > 0 ? max(0, c.pos - a.window + 1) : 0;
-  c.wave_lo = a.window > 0 ? max(0, pos0 - a.window + 1) : 0;
+  c.lo = first_visible(a, c.pos);
+  c.wave_lo = first_visible(a, pos0);
   const int tile_lo = c.wave_lo / TILE_KEYS, tile_hi = (pos0 + nvalid - 1) / TILE_KEYS;
 
   frag_t qf[NQS];
@@ -595,7 +603,7 @@ __global__ __launch_bounds__(64 * NW, EXT ? 1 : 2) void attn_prefill_lds_kernel(
   const int k_len = a.k_len[seq];
   const int rows_item = min(ROWS_WG, q_len - q_off0);    // this workgroup's rows
   const int pos_item = k_len - q_len + q_off0;           // position of the item's first row
-  const int item_lo = a.window > 0 ? max(0, pos_item - a.window + 1) : 0;
+  const int item_lo = first_visible(a, pos_item);
   const int tile_lo = item_lo / TILE_KEYS, tile_hi = (pos_item + rows_item - 1) / TILE_KEYS;
   // The tiles this workgroup walks: with kept first keys, their tiles (those that lie before the window's) and then the
   // window's; otherwise tile_lo .. tile_hi.
@@ -608,11 +616,11 @@ __global__ __launch_bounds__(64 * NW, EXT ? 1 : 2) void attn_prefill_lds_kernel(
   // ---- this wave's rows ----
   const int rows_wave = min(16, rows_item - 16 * wave);  // <= 0: the wave only helps to load
   const int pos_wave = pos_item + 16 * wave;
-  const int wave_lo = a.window > 0 ? max(0, pos_wave - a.window + 1) : 0;
+  const int wave_lo = first_visible(a, pos_wave);
   const int wtile_lo = wave_lo / TILE_KEYS, wtile_hi = rows_wave > 0 ? (pos_wave + rows_wave - 1) / TILE_KEYS : -1;
   const bool row_ok = r16 < rows_wave;
   const int pos = pos_wave + r16;
-  const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
+  const int lo = first_visible(a, pos);
   const int tok = q_begin + q_off0 + 16 * wave + r16;
   frag_t qf[NQS];
   load_q<NQS>(a, tok, head, row_ok, g, qf);
@@ -707,7 +715,7 @@ __global__ __launch_bounds__(64 * NW, EXT ? 1 : 2) void attn_prefill_lds_kernel(
       __builtin_amdgcn_sched_barrier(0);
       // ---- the row's new maximum, its probabilities, its sums so far under the new maximum ----
       const bool full = rows_wave >= 16 && kb + TILE_KEYS - 1 <= pos_wave &&
-                        kb >= (a.window > 0 ? max(0, pos_wave + 15 - a.window + 1) : 0);
+                        kb >= (first_visible(a, pos_wave + 15));
       frag_t pf[EXT ? P_PARTS : 1][KEY_SLABS];
       float ca;
       const bool fresh = !(Ms > -INFINITY);
@@ -813,7 +821,7 @@ __global__ __launch_bounds__(64 * PLAIN_WAVES) void attn_decode_plain_kernel(Att
   const int k_len = a.k_len[seq];
   const int tok = q_begin + q_off;
   const int pos = k_len - q_len + q_off;
-  const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
+  const int lo = first_visible(a, pos);
   const int t0 = max(lo / TILE_KEYS, seg * SEG_TILES), t1 = min(pos / TILE_KEYS, seg * SEG_TILES + SEG_TILES - 1);
   if (t0 > t1) return;   // whole wave; no barrier follows
 
@@ -865,7 +873,7 @@ __global__ __launch_bounds__(64 * SEG_WAVES, 2) void attn_decode_seg_kernel(Attn
   const int k_len = a.k_len[seq];
   const int tok = q_begin + q_off;
   const int pos = k_len - q_len + q_off;
-  const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
+  const int lo = first_visible(a, pos);
   const int t0 = max(lo / TILE_KEYS, seg * SEG_TILES), t1 = min(pos / TILE_KEYS, seg * SEG_TILES + SEG_TILES - 1);
   if (t0 > t1) return;   // whole wave; no barrier follows
 
@@ -946,7 +954,7 @@ __global__ __launch_bounds__(128, 2) void attn_decode_pair_kernel(AttnArgs a) {
   const int k_len = a.k_len[seq];
   const int tok = q_begin + q_off;
   const int pos = k_len - q_len + q_off;
-  const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
+  const int lo = first_visible(a, pos);
   const int s0 = max(lo / TILE_KEYS, seg * SEG_TILES), s1 = min(pos / TILE_KEYS, seg * SEG_TILES + SEG_TILES - 1);
   if (s0 > s1) return;                                  // the whole workgroup
   const int n = s1 - s0 + 1, n_first = (n + 1) >> 1;
@@ -1089,8 +1097,8 @@ __global__ __launch_bounds__(256) void attn_prefill_ext_kernel(AttnArgs a, int h
   const int tok = q_begin + q_off + c.r16;
   const int pos0 = k_len - q_len + q_off;
   c.pos = pos0 + c.r16;
-  c.lo = a.window > 0 ? max(0, c.pos - a.window + 1) : 0;
-  c.wave_lo = a.window > 0 ? max(0, pos0 - a.window + 1) : 0;
+  c.lo = first_visible(a, c.pos);
+  c.wave_lo = first_visible(a, pos0);
   c.keep = a.window > 0 ? a.keep : 0;
   const int keep_tiles = (c.keep + TILE_KEYS - 1) / TILE_KEYS;
   const int tile_lo = c.wave_lo / TILE_KEYS, tile_hi = (pos0 + nvalid - 1) / TILE_KEYS;
@@ -1143,7 +1151,7 @@ __global__ __launch_bounds__(64 * PLAIN_WAVES) void attn_decode_ext_kernel(AttnA
   const int k_len = a.k_len[seq];
   const int tok = q_begin + q_off;
   const int pos = k_len - q_len + q_off;
-  const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
+  const int lo = first_visible(a, pos);
   const int keep = a.window > 0 ? a.keep : 0;
   const int keep_tiles = (keep + TILE_KEYS - 1) / TILE_KEYS, tile_lo = lo / TILE_KEYS;
   const int t0 = seg * SEG_TILES, t1 = min(pos / TILE_KEYS, seg * SEG_TILES + SEG_TILES - 1);
@@ -1196,7 +1204,7 @@ __global__ __launch_bounds__(64 * SEG_WAVES, 2) void attn_decode_seg_ext_kernel(
   const int k_len = a.k_len[seq];
   const int tok = q_begin + q_off;
   const int pos = k_len - q_len + q_off;
-  const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
+  const int lo = first_visible(a, pos);
   const int keep = a.window > 0 ? a.keep : 0;
   const int keep_tiles = (keep + TILE_KEYS - 1) / TILE_KEYS, tile_lo = lo / TILE_KEYS;
   // The segment's tiles that hold visible keys, as a mask of SEG_TILES bits.
@@ -1270,7 +1278,7 @@ __global__ __launch_bounds__(64) void attn_combine_kernel(AttnArgs a) {
   const int k_len = a.k_len[seq];
   const int tok = q_begin + q_off;
   const int pos = k_len - q_len + q_off;
-  const int lo = a.window > 0 ? max(0, pos - a.window + 1) : 0;
+  const int lo = first_visible(a, pos);
   // Segments that hold kept first keys come before the window's; those in between were not computed.
   const int keep_tiles = a.window > 0 ? (a.keep + TILE_KEYS - 1) / TILE_KEYS : 0, tile_lo = lo / TILE_KEYS;
   const int seg_begin = keep_tiles > 0 ? 0 : lo / (TILE_KEYS * SEG_TILES), seg_end = pos / (TILE_KEYS * SEG_TILES) + 1;
@@ -1508,11 +1516,12 @@ int vk_paged_attention(elem_t* out, const elem_t* q, const elem_t* kc, const ele
 // The attention with capped scores, kept first keys, a sink and unrounded weights (see "Capped scores" above).
 // mode 0: items of prompt rows; mode 1: items of one decoded token each, with nseg and scratch as vk_paged_attention
 // takes them.  keep > 0 needs a window.  softcap 0: no cap.  sinks: [nq] elements (or floats with sinks_f32) or null.
-int vk_paged_attention_capped(elem_t* out, const elem_t* q, const elem_t* kc, const elem_t* vc, const int32_t* block_table,
-                              int bt_stride, const int32_t* cu_q, const int32_t* k_len, const int32_t* items, int n_items, int mode,
-                              int nseg, float* scratch, int total_tokens, int nq, int nkv, int d, int P, int window, int keep,
-                              float scale, float softcap, const void* sinks, int sinks_f32, hipStream_t st) {
+static int attention_capped_launch(elem_t* out, const elem_t* q, const elem_t* kc, const elem_t* vc, const int32_t* block_table,
+                                   int bt_stride, const int32_t* cu_q, const int32_t* k_len, const int32_t* items, int n_items, int mode,
+                                   int nseg, float* scratch, int total_tokens, int nq, int nkv, int d, int P, int window, int keep, int block,
+                                   float scale, float softcap, const void* sinks, int sinks_f32, hipStream_t st) {
   (void)total_tokens;
+  VK_REQUIRE(block >= 0 && (block == 0 || window == 0), "attention: blocks of positions (%d) and a window (%d) exclude each other", block, window);
   VK_REQUIRE(nq > 0 && nkv > 0 && nq % nkv == 0, "attention: %d q heads are not a multiple of %d kv heads", nq, nkv);
   VK_REQUIRE(d >= 16 && d <= 256 && d % 16 == 0, "attention: head size %d must be a multiple of 16 in 16..256", d);
   VK_REQUIRE(P >= 8 && (P & (P - 1)) == 0, "attention: page size %d must be a power of two >= 8", P);
@@ -1526,7 +1535,7 @@ int vk_paged_attention_capped(elem_t* out, const elem_t* q, const elem_t* kc, co
   a.items = items; a.bt_stride = bt_stride; a.nq = nq; a.nkv = nkv; a.d = d; a.P = P; a.window = window;
   a.nseg = nseg; a.scale_log2 = scale * LOG2E;
   a.part_ml = nullptr; a.part_acc = nullptr;
-  a.keep = keep; a.scale = scale; a.softcap = softcap; a.sinks = sinks; a.sinks_f32 = sinks_f32;
+  a.keep = keep; a.scale = scale; a.softcap = softcap; a.sinks = sinks; a.sinks_f32 = sinks_f32; a.block = block;
   const int G = nq / nkv;
   if (mode == 0 && vk_attn_prefill_shares_tiles(d, P)) {
     // Key and value tiles through LDS, as for the plain attention; eight waves a workgroup unless they are few.
@@ -1595,6 +1604,26 @@ int vk_paged_attention_capped(elem_t* out, const elem_t* q, const elem_t* kc, co
   if (vk_check_launch("attention (decoded rows, capped scores)")) return 1;
   attn_combine_kernel<<<dim3(n_items, nq), 64, 0, st>>>(a);
   return vk_check_launch("attention (combine)");
+}
+
+int vk_paged_attention_capped(elem_t* out, const elem_t* q, const elem_t* kc, const elem_t* vc, const int32_t* block_table,
+                              int bt_stride, const int32_t* cu_q, const int32_t* k_len, const int32_t* items, int n_items, int mode,
+                              int nseg, float* scratch, int total_tokens, int nq, int nkv, int d, int P, int window, int keep,
+                              float scale, float softcap, const void* sinks, int sinks_f32, hipStream_t st) {
+  return attention_capped_launch(out, q, kc, vc, block_table, bt_stride, cu_q, k_len, items, n_items, mode, nseg, scratch, total_tokens, nq, nkv,
+                                 d, P, window, keep, 0, scale, softcap, sinks, sinks_f32, st);
+}
+
+// The same kernels with positions cut into blocks of `block`: the row at position p sees key j <= p only if
+// j / block == p / block (integer division), counted from the sequence's first position.  The arithmetic and the
+// order of the tiles are those of a window whose first key is the start of p's block.
+int vk_paged_attention_blocked(elem_t* out, const elem_t* q, const elem_t* kc, const elem_t* vc, const int32_t* block_table,
+                               int bt_stride, const int32_t* cu_q, const int32_t* k_len, const int32_t* items, int n_items, int mode,
+                               int nseg, float* scratch, int total_tokens, int nq, int nkv, int d, int P, int block,
+                               float scale, float softcap, const void* sinks, int sinks_f32, hipStream_t st) {
+  VK_REQUIRE(block > 0, "attention: a block of %d positions", block);
+  return attention_capped_launch(out, q, kc, vc, block_table, bt_stride, cu_q, k_len, items, n_items, mode, nseg, scratch, total_tokens, nq, nkv,
+                                 d, P, 0, 0, block, scale, softcap, sinks, sinks_f32, st);
 }
 
 }  // extern "C"

@@ -24,14 +24,15 @@ __global__ __launch_bounds__(256) void delta_conv_kernel(float* __restrict__ y, 
                                                          const elem_t* __restrict__ taps, const float* __restrict__ state,
                                                          int64_t state_stride, int64_t tail_offset, const int32_t* __restrict__ token_seq,
                                                          const int32_t* __restrict__ cu_q, const int32_t* __restrict__ positions,
-                                                         const int32_t* __restrict__ slots, int C, int K) {
+                                                         const int32_t* __restrict__ slots, int C, int K,
+                                                         const elem_t* __restrict__ bias) {
   const int t = blockIdx.x;
   const int s = token_seq[t];
   const int first = cu_q[s], i = t - first;
   const bool fresh = positions[first] == 0;
   const float* tail = state + (int64_t)slots[s] * state_stride + tail_offset;
   for (int c = blockIdx.y * blockDim.x + threadIdx.x; c < C; c += gridDim.y * blockDim.x) {
-    float acc = 0.f;
+    float acc = bias != nullptr ? to_f32(bias[c]) : 0.f;
     for (int j = 0; j < K; ++j) {
       const int li = i - (K - 1) + j;
       float v;
@@ -348,22 +349,37 @@ int vk_delta_lanes_per_column(int d) {
   return R;
 }
 
-// y [T, C] floats from the columns x[:, 0:C] of rows of length ldx; then the tails are moved on.
-int vk_delta_conv(float* y, const elem_t* x, int64_t ldx, const elem_t* taps, float* state, int64_t state_stride, int64_t tail_offset,
-                  const int32_t* token_seq, const int32_t* cu_q, const int32_t* positions, const int32_t* slots, int T, int S, int C, int K,
-                  hipStream_t st) {
+// y [T, C] floats from the columns x[:, 0:C] of rows of length ldx; then the tails are moved on.  bias: [C] or null, what
+// every channel's sum starts from.
+static int conv_launch(float* y, const elem_t* x, int64_t ldx, const elem_t* taps, const elem_t* bias, float* state, int64_t state_stride,
+                       int64_t tail_offset, const int32_t* token_seq, const int32_t* cu_q, const int32_t* positions, const int32_t* slots, int T,
+                       int S, int C, int K, hipStream_t st) {
   VK_REQUIRE(T >= 0 && S >= 0 && C > 0 && K >= 1 && K <= DELTA_MAX_TAPS + 1, "short convolution: bad sizes T=%d C=%d taps=%d (at most %d)", T, C, K,
              DELTA_MAX_TAPS + 1);
   VK_REQUIRE(ldx >= C && tail_offset >= 0 && state_stride >= tail_offset + (int64_t)(K - 1) * C, "short convolution: the state does not hold the tails");
   if (T == 0 || S == 0) return 0;
   const int by = (C + 255) / 256 < 64 ? (C + 255) / 256 : 64;
-  delta_conv_kernel<<<dim3(T, by), 256, 0, st>>>(y, x, ldx, taps, state, state_stride, tail_offset, token_seq, cu_q, positions, slots, C, K);
+  delta_conv_kernel<<<dim3(T, by), 256, 0, st>>>(y, x, ldx, taps, state, state_stride, tail_offset, token_seq, cu_q, positions, slots, C, K, bias);
   if (vk_check_launch("short convolution")) return 1;
   if (K > 1) {
     delta_conv_tail_kernel<<<dim3(S, by), 256, 0, st>>>(x, ldx, state, state_stride, tail_offset, cu_q, positions, slots, C, K);
     return vk_check_launch("short convolution (tails)");
   }
   return 0;
+}
+
+int vk_delta_conv(float* y, const elem_t* x, int64_t ldx, const elem_t* taps, float* state, int64_t state_stride, int64_t tail_offset,
+                  const int32_t* token_seq, const int32_t* cu_q, const int32_t* positions, const int32_t* slots, int T, int S, int C, int K,
+                  hipStream_t st) {
+  return conv_launch(y, x, ldx, taps, nullptr, state, state_stride, tail_offset, token_seq, cu_q, positions, slots, T, S, C, K, st);
+}
+
+// The same with a bias per channel.
+int vk_delta_conv_bias(float* y, const elem_t* x, int64_t ldx, const elem_t* taps, const elem_t* bias, float* state, int64_t state_stride,
+                       int64_t tail_offset, const int32_t* token_seq, const int32_t* cu_q, const int32_t* positions, const int32_t* slots, int T,
+                       int S, int C, int K, hipStream_t st) {
+  VK_REQUIRE(bias != nullptr, "short convolution: the bias is missing");
+  return conv_launch(y, x, ldx, taps, bias, state, state_stride, tail_offset, token_seq, cu_q, positions, slots, T, S, C, K, st);
 }
 
 int vk_delta_unit(float* x, int64_t ld, int col0, int T, int heads, int d, float eps, float scale, hipStream_t st) {

@@ -113,9 +113,24 @@ struct Kernels::Fn {
   int (*delta_prep)(P, int64_t, int, int, int, int, int, int, float, float, P, CP, CP, CP, int, hipStream_t);
   int (*delta_rule)(P, CP, int64_t, int, int, int, CP, CP, int64_t, P, int64_t, CP, CP, CP, int, int, int, int, int, hipStream_t);
   int (*delta_out)(P, int64_t, CP, CP, int64_t, CP, int, int, int, int, float, hipStream_t);
+  int (*delta_conv_bias)(P, CP, int64_t, CP, CP, P, int64_t, int64_t, CP, CP, CP, CP, int, int, int, int, hipStream_t);
+  int (*paged_attention_blocked)(P, CP, CP, CP, CP, int, CP, CP, CP, int, int, int, P, int, int, int, int, int, int, float, float, CP, int,
+                                 hipStream_t);
+  int (*qkv_post_angles)(CP, int64_t, P, P, P, CP, float, int, CP, CP, int, int, int, int, int, hipStream_t);
+  int (*embed_scaled)(P, CP, CP, int, int, int, float, hipStream_t);
+  int (*stream_add)(P, CP, CP, int, CP, int, int64_t, hipStream_t);
+  int (*stream_pair_norm)(P, CP, CP, CP, CP, int, int, int, float, float, float, hipStream_t);
+  int (*ssm_scan)(P, CP, int64_t, int, int, CP, int64_t, CP, CP, CP, int, P, int64_t, CP, CP, CP, int, int, int, int, int, hipStream_t);
+  int (*ssm_gate_norm)(P, int64_t, CP, CP, int64_t, CP, int, int, int, int, float, hipStream_t);
+  int (*moe_max_tiles)(int, int, int);
+  int (*moe_route)(P, P, CP, CP, int, int, int, int, float, hipStream_t);
+  int (*moe_plan)(CP, P, P, P, int, int, int, hipStream_t);
+  int (*moe_up)(P, int64_t, CP, int64_t, CP, CP, CP, int, int, int, int, int, hipStream_t);
+  int (*moe_down)(P, CP, int64_t, CP, CP, CP, int, int, int, int, int, hipStream_t);
+  int (*moe_combine)(P, CP, CP, CP, int, int, int, hipStream_t);
 };
 
-static constexpr int KERNEL_ABI = 15;
+static constexpr int KERNEL_ABI = 16;
 
 Kernels::Kernels(const std::string& lib_dir, const std::string& name) : name_(name), fn_(new Fn) {
   if (name == "bf16") dtype_ = DType::BF16;
@@ -145,7 +160,11 @@ Kernels::Kernels(const std::string& lib_dir, const std::string& name) : name_(na
   VK(stream_mix, "vk_stream_mix"); VK(gather_rows_f32, "vk_gather_rows_f32"); VK(softcap, "vk_softcap");
   VK(qkv_post_bias, "vk_qkv_post_bias"); VK(paged_attention_capped, "vk_paged_attention_capped");
   VK(delta_conv, "vk_delta_conv"); VK(delta_prep, "vk_delta_prep"); VK(delta_unit, "vk_delta_unit"); VK(delta_decay, "vk_delta_decay"); VK(delta_rule, "vk_delta_rule");
-  VK(delta_out, "vk_delta_out");
+  VK(delta_out, "vk_delta_out"); VK(delta_conv_bias, "vk_delta_conv_bias"); VK(paged_attention_blocked, "vk_paged_attention_blocked");
+  VK(qkv_post_angles, "vk_qkv_post_angles"); VK(embed_scaled, "vk_embed_scaled"); VK(stream_add, "vk_stream_add");
+  VK(stream_pair_norm, "vk_stream_pair_norm"); VK(ssm_scan, "vk_ssm_scan"); VK(ssm_gate_norm, "vk_ssm_gate_norm");
+  VK(moe_max_tiles, "vk_moe_max_tiles"); VK(moe_route, "vk_moe_route"); VK(moe_plan, "vk_moe_plan"); VK(moe_up, "vk_moe_up");
+  VK(moe_down, "vk_moe_down"); VK(moe_combine, "vk_moe_combine");
 #undef VK
   segment_keys_ = fn_->attn_segment_keys();
   item_rows_ = fn_->attn_item_rows();
@@ -490,9 +509,10 @@ Tensor Kernels::qkv_post_bias(const Tensor& qkv, int nq, int nkv, int d, const T
 
 void Kernels::paged_attention_capped(Tensor& out, const Tensor& q, const Tensor& k_cache, const Tensor& v_cache, const Tensor& block_table,
                                      const Tensor& cu_q, const Tensor& k_len, const Tensor& items, int mode, float scale, int window, int keep,
-                                     float softcap, const Tensor* sinks, int max_k_len, int nseg, const Tensor* scratch) {
+                                     float softcap, const Tensor* sinks, int max_k_len, int nseg, const Tensor* scratch, int block) {
   expect(q, "q", dtype_);
   expect(block_table, "block table", DType::I32);
+  if (block < 0 || (block > 0 && (window != 0 || keep != 0))) throw EngineError("attention: blocks of positions exclude a window");
   if (q.shape.size() != 3 || k_cache.shape.size() != 4 || block_table.shape.size() != 2)
     throw EngineError("attention: q " + q.describe() + ", k cache " + k_cache.describe() + ", block table " + block_table.describe());
   const int64_t T = q.dim(0), nq = q.dim(1), d = q.dim(2), pages = k_cache.dim(0), nkv = k_cache.dim(1), P = k_cache.dim(2);
@@ -520,6 +540,12 @@ void Kernels::paged_attention_capped(Tensor& out, const Tensor& q, const Tensor&
       throw EngineError("attention: scratch of " + std::to_string(need) + " floats needed");
     sp = scratch->data;
   }
+  if (block > 0) {
+    call(fn_->paged_attention_blocked(out.data, q.data, k_cache.data, v_cache.data, block_table.data, (int)W, cu_q.data, k_len.data, items.data,
+                                      (int)n_items, mode, nseg, sp, (int)T, (int)nq, (int)nkv, (int)d, (int)P, block, scale, softcap,
+                                      sinks ? sinks->data : nullptr, sf, stream));
+    return;
+  }
   call(fn_->paged_attention_capped(out.data, q.data, k_cache.data, v_cache.data, block_table.data, (int)W, cu_q.data, k_len.data, items.data,
                                    (int)n_items, mode, nseg, sp, (int)T, (int)nq, (int)nkv, (int)d, (int)P, window, keep, scale, softcap,
                                    sinks ? sinks->data : nullptr, sf, stream));
@@ -527,11 +553,11 @@ void Kernels::paged_attention_capped(Tensor& out, const Tensor& q, const Tensor&
 
 // ------------------------------------------------------------------------------------- the delta rule
 Tensor Kernels::delta_conv(const Tensor& x, const Tensor& taps, Tensor& state, int64_t tail_offset, const Tensor& token_seq, const Tensor& cu_q,
-                           const Tensor& positions, const Tensor& slots) {
+                           const Tensor& positions, const Tensor& slots, int64_t first_col, const Tensor* bias) {
   expect(x, "convolution input", dtype_);
   expect(taps, "convolution taps", dtype_);
   expect(state, "state", DType::F32);
-  if (x.shape.size() != 2 || taps.shape.size() != 2 || state.shape.size() != 2 || taps.dim(0) > x.dim(1))
+  if (x.shape.size() != 2 || taps.shape.size() != 2 || state.shape.size() != 2 || first_col < 0 || first_col + taps.dim(0) > x.dim(1))
     throw EngineError("short convolution: input " + x.describe() + ", taps " + taps.describe() + ", state " + state.describe());
   const int64_t T = x.dim(0), C = taps.dim(0), K = taps.dim(1), S = slots.numel();
   expect(token_seq, "token sequences", DType::I32, {T});
@@ -539,7 +565,14 @@ Tensor Kernels::delta_conv(const Tensor& x, const Tensor& taps, Tensor& state, i
   expect(cu_q, "cu_q", DType::I32, {S + 1});
   expect(slots, "state slots", DType::I32, {S});
   Tensor y = empty({T, C}, DType::F32);
-  call(fn_->delta_conv(y.data, x.data, x.dim(1), taps.data, state.data, state.dim(1), tail_offset, token_seq.data, cu_q.data, positions.data,
+  const void* x0 = static_cast<const char*>(x.data) + (size_t)first_col * dtype_bytes(dtype_);
+  if (bias) {
+    expect(*bias, "convolution bias", dtype_, {C});
+    call(fn_->delta_conv_bias(y.data, x0, x.dim(1), taps.data, bias->data, state.data, state.dim(1), tail_offset, token_seq.data, cu_q.data,
+                              positions.data, slots.data, (int)T, (int)S, (int)C, (int)K, stream));
+    return y;
+  }
+  call(fn_->delta_conv(y.data, x0, x.dim(1), taps.data, state.data, state.dim(1), tail_offset, token_seq.data, cu_q.data, positions.data,
                        slots.data, (int)T, (int)S, (int)C, (int)K, stream));
   return y;
 }
@@ -605,6 +638,150 @@ Tensor Kernels::delta_out(const Tensor& o, const Tensor& gate, const Tensor& w, 
   Tensor y = empty({o.dim(0), width});
   call(fn_->delta_out(y.data, width, o.data, gate.data, gate.dim(1), w.data, wf, (int)o.dim(0), H, dv, eps, stream));
   return y;
+}
+
+// ---------------------------------------------------- scaled embedding, sums and means of branches
+Tensor Kernels::embed_scaled(const Tensor& table, const Tensor& ids, float scale) {
+  expect(table, "embedding table", dtype_);
+  if (table.shape.size() != 2) throw EngineError("embedding table is " + table.describe());
+  const int64_t V = table.dim(0), H = table.dim(1), T = ids.numel();
+  expect(ids, "ids", DType::I32, {T});
+  Tensor out = empty({T, H}, DType::F32);
+  call(fn_->embed_scaled(out.data, table.data, ids.data, (int)T, (int)H, (int)V, scale, stream));
+  return out;
+}
+
+void Kernels::stream_add(Tensor& s, const Tensor& a, const Tensor* b) {
+  expect(s, "stream", DType::F32);
+  for (const Tensor* t : {&a, b}) {
+    if (!t) continue;
+    if (t->dtype != DType::F32) expect(*t, "a branch's output", dtype_, s.shape);
+    else expect(*t, "a branch's output", DType::F32, s.shape);
+  }
+  call(fn_->stream_add(s.data, s.data, a.data, a.dtype == DType::F32 ? 1 : 0, b ? b->data : nullptr, b && b->dtype == DType::F32 ? 1 : 0, s.numel(),
+                       stream));
+}
+
+Tensor Kernels::stream_pair_norm(const Tensor& a, const Tensor& wa, const Tensor& b, const Tensor& wb, float eps, float ca, float cb) {
+  expect(a, "first branch", dtype_);
+  if (a.shape.size() != 2) throw EngineError("pair norm: the first branch is " + a.describe());
+  expect(b, "second branch", dtype_, a.shape);
+  const int wf = norm_weight(wa, "first branch's norm weight", a.dim(1));
+  if (norm_weight(wb, "second branch's norm weight", a.dim(1)) != wf) throw EngineError("pair norm: the two weights must have one type");
+  Tensor out = empty(a.shape, DType::F32);
+  call(fn_->stream_pair_norm(out.data, a.data, wa.data, b.data, wb.data, wf, (int)a.dim(0), (int)a.dim(1), eps, ca, cb, stream));
+  return out;
+}
+
+Tensor Kernels::qkv_post_angles(const Tensor& qkv, int nq, int nkv, int d, const Tensor* k_cache, const Tensor* v_cache, int page_size,
+                                const Tensor& inv_freq, float mag, const Tensor& positions, const Tensor* slots) {
+  expect(qkv, "qkv", dtype_);
+  const int64_t W = (int64_t)(nq + 2 * nkv) * d;
+  if (qkv.shape.size() != 2 || qkv.dim(1) != W) throw EngineError("qkv_post: rows are " + qkv.describe() + ", expected width " + std::to_string(W));
+  const int64_t T = qkv.dim(0);
+  expect(inv_freq, "rotation frequencies", DType::F32);
+  if (inv_freq.shape.size() != 1 || inv_freq.dim(0) < 1 || 2 * inv_freq.dim(0) > d)
+    throw EngineError("qkv_post: rotation frequencies are " + inv_freq.describe() + " for a head size of " + std::to_string(d));
+  expect(positions, "positions", DType::I32, {T});
+  Tensor q_out;
+  if (nq) q_out = empty({T, nq, d});
+  if (nkv) {
+    if (!k_cache || !v_cache || !slots) throw EngineError("qkv_post: a store needs both caches and slots");
+    if (k_cache->shape.size() != 4) throw EngineError("k cache is " + k_cache->describe());
+    const int64_t pages = k_cache->dim(0);
+    expect(*k_cache, "k cache", dtype_, {pages, nkv, page_size, d});
+    expect(*v_cache, "v cache", dtype_, {pages, nkv, d, page_size});
+    expect(*slots, "slots", DType::I32, {T});
+  }
+  call(fn_->qkv_post_angles(qkv.data, W, nq ? q_out.data : nullptr, nkv ? k_cache->data : nullptr, nkv ? v_cache->data : nullptr, inv_freq.data, mag,
+                            (int)inv_freq.dim(0), positions.data, nkv ? slots->data : nullptr, (int)T, nq, nkv, d, page_size, stream));
+  return q_out;
+}
+
+// ---------------------------------------------------------------------------- state-space recurrence
+Tensor Kernels::ssm_scan(const Tensor& xbc, int64_t b_col, int64_t c_col, const Tensor& proj, int64_t dt_col, const Tensor& dt_bias,
+                         const Tensor& A_log, const Tensor& D, Tensor& state, const Tensor& cu_q, const Tensor& positions, const Tensor& slots, int H,
+                         int G, int N, int P) {
+  expect(xbc, "state-space input", DType::F32);
+  expect(proj, "input projection", dtype_);
+  expect(state, "state", DType::F32);
+  if (xbc.shape.size() != 2 || proj.shape.size() != 2 || state.shape.size() != 2 || proj.dim(0) != xbc.dim(0) || dt_col < 0 ||
+      dt_col + H > proj.dim(1) || b_col < (int64_t)H * P || c_col < 0 || std::max(b_col, c_col) + (int64_t)G * N > xbc.dim(1) ||
+      state.dim(1) < (int64_t)H * P * N)
+    throw EngineError("state-space scan: input " + xbc.describe() + ", projection " + proj.describe() + ", state " + state.describe());
+  const int64_t T = xbc.dim(0), S = slots.numel();
+  const int wf = norm_weight(dt_bias, "dt_bias", H);
+  if (norm_weight(A_log, "A_log", H) != wf || norm_weight(D, "D", H) != wf) throw EngineError("state-space scan: dt_bias, A_log and D must have one type");
+  expect(positions, "positions", DType::I32, {T});
+  expect(cu_q, "cu_q", DType::I32, {S + 1});
+  expect(slots, "state slots", DType::I32, {S});
+  Tensor y = empty({T, H, P}, DType::F32);
+  call(fn_->ssm_scan(y.data, xbc.data, xbc.dim(1), (int)b_col, (int)c_col, static_cast<const char*>(proj.data) + (size_t)dt_col * dtype_bytes(dtype_),
+                     proj.dim(1), dt_bias.data, A_log.data, D.data, wf, state.data, state.dim(1), cu_q.data, positions.data, slots.data, (int)S, H, G,
+                     N, P, stream));
+  return y;
+}
+
+Tensor Kernels::ssm_gate_norm(const Tensor& y, const Tensor& proj, int64_t z_col, const Tensor& w, int parts, float eps, int64_t width) {
+  expect(y, "state-space read-out", DType::F32);
+  expect(proj, "input projection", dtype_);
+  if (y.shape.size() < 2 || proj.shape.size() != 2 || proj.dim(0) != y.dim(0)) throw EngineError("gated norm: " + y.describe() + " with " + proj.describe());
+  const int64_t T = y.dim(0), inner = T ? y.numel() / T : 0;
+  if (inner <= 0 || parts <= 0 || inner % parts || z_col < 0 || z_col + inner > proj.dim(1) || width < inner)
+    throw EngineError("gated norm: rows of " + std::to_string(inner) + " in " + std::to_string(parts) + " parts");
+  const int wf = norm_weight(w, "read-out norm weight", inner);
+  Tensor out = empty({T, width});
+  call(fn_->ssm_gate_norm(out.data, width, y.data, static_cast<const char*>(proj.data) + (size_t)z_col * dtype_bytes(dtype_), proj.dim(1), w.data, wf,
+                          (int)T, (int)inner, parts, eps, stream));
+  return out;
+}
+
+// ------------------------------------------------------------------------------ mixture of experts
+Kernels::MoePlan Kernels::moe_route(const Tensor& h, const Tensor& router, int top, float weight_eps) {
+  expect(h, "router input", dtype_);
+  expect(router, "router weight", dtype_);
+  if (h.shape.size() != 2 || router.shape.size() != 2 || router.dim(1) != h.dim(1) || top < 1 || top > router.dim(0))
+    throw EngineError("router: input " + h.describe() + ", weight " + router.describe() + ", top " + std::to_string(top));
+  const int64_t T = h.dim(0), E = router.dim(0);
+  MoePlan p;
+  p.top = top;
+  p.experts = (int)E;
+  const int64_t tiles = fn_->moe_max_tiles((int)T, top, (int)E);
+  p.idx = empty({T, top}, DType::I32);
+  p.wts = empty({T, top}, DType::F32);
+  p.row_pair = empty({tiles * 16}, DType::I32);
+  p.pair_row = empty({T * top}, DType::I32);
+  p.tile_expert = empty({tiles}, DType::I32);
+  call(fn_->moe_route(p.idx.data, p.wts.data, h.data, router.data, (int)T, (int)h.dim(1), (int)E, top, weight_eps, stream));
+  call(fn_->moe_plan(p.idx.data, p.row_pair.data, p.pair_row.data, p.tile_expert.data, (int)T, top, (int)E, stream));
+  return p;
+}
+
+Tensor Kernels::moe_up(const Tensor& h, const Tensor& w_up, const MoePlan& plan) {
+  expect(h, "experts' input", dtype_);
+  expect(w_up, "experts' up weights", dtype_);
+  if (h.shape.size() != 2 || w_up.shape.size() != 3 || w_up.dim(0) != plan.experts || w_up.dim(2) != h.dim(1) || plan.idx.dim(0) != h.dim(0))
+    throw EngineError("experts (up): input " + h.describe() + ", weights " + w_up.describe());
+  const int64_t T = h.dim(0), N = w_up.dim(1);
+  Tensor act = empty({plan.row_pair.dim(0), N});
+  call(fn_->moe_up(act.data, N, h.data, h.dim(1), w_up.data, plan.row_pair.data, plan.tile_expert.data, (int)T, plan.top, plan.experts, (int)N,
+                   (int)h.dim(1), stream));
+  return act;
+}
+
+Tensor Kernels::moe_down_sum(const Tensor& act, const Tensor& w_down, const MoePlan& plan, int64_t T) {
+  expect(act, "experts' activations", dtype_);
+  expect(w_down, "experts' down weights", dtype_);
+  if (act.shape.size() != 2 || w_down.shape.size() != 3 || w_down.dim(0) != plan.experts || w_down.dim(2) != act.dim(1) ||
+      act.dim(0) != plan.row_pair.dim(0) || plan.idx.dim(0) != T)
+    throw EngineError("experts (down): activations " + act.describe() + ", weights " + w_down.describe());
+  const int64_t W = w_down.dim(1);
+  Tensor y = empty({act.dim(0), W}, DType::F32);
+  call(fn_->moe_down(y.data, act.data, act.dim(1), w_down.data, plan.row_pair.data, plan.tile_expert.data, (int)T, plan.top, plan.experts, (int)W,
+                     (int)act.dim(1), stream));
+  Tensor out = empty({T, W}, DType::F32);
+  call(fn_->moe_combine(out.data, y.data, plan.wts.data, plan.pair_row.data, (int)T, (int)W, plan.top, stream));
+  return out;
 }
 
 int Kernels::sample_scratch_words(int rows) const { return fn_->sample_scratch_words(rows); }

@@ -150,14 +150,16 @@ class Kernels {
   // qkv_post with a bias [(nq + 2 nkv) d] added to the rows first.
   Tensor qkv_post_bias(const Tensor& qkv, int nq, int nkv, int d, const Tensor* k_cache, const Tensor* v_cache, int page_size,
                        const Tensor* slots, const Tensor& bias);
-  // Attention with capped scores, kept first keys, a sink per head and unrounded weights (attention.hip).
+  // Attention with capped scores, kept first keys, a sink per head and unrounded weights (attention.hip).  block > 0
+  // (without a window): positions are cut into blocks of that many, and a row sees the keys of its own block only.
   void paged_attention_capped(Tensor& out, const Tensor& q, const Tensor& k_cache, const Tensor& v_cache, const Tensor& block_table,
                               const Tensor& cu_q, const Tensor& k_len, const Tensor& items, int mode, float scale, int window, int keep,
-                              float softcap, const Tensor* sinks, int max_k_len, int nseg, const Tensor* scratch);
+                              float softcap, const Tensor* sinks, int max_k_len, int nseg, const Tensor* scratch, int block = 0);
   // ---- the gated delta rule with a decay per key channel (delta.hip)
   // silu(short causal convolution) of the first taps.dim(0) columns of x, floats [T, C]; the state's tails move on.
+  // first_col: where the convolution's channels start in x's rows; bias: [channels] or null.
   Tensor delta_conv(const Tensor& x, const Tensor& taps, Tensor& state, int64_t tail_offset, const Tensor& token_seq, const Tensor& cu_q,
-                    const Tensor& positions, const Tensor& slots);
+                    const Tensor& positions, const Tensor& slots, int64_t first_col = 0, const Tensor* bias = nullptr);
   void delta_unit(Tensor& x, int64_t col0, int heads, int d, float eps, float scale);
   Tensor delta_decay(const Tensor& a, const Tensor& dt_bias, const Tensor& A_log, int H, int d);
   // Both unit norms (q at q_col times q_scale, k at k_col; G heads of d each) and the decays, in one launch; returns the decays.
@@ -167,6 +169,35 @@ class Kernels {
                     const Tensor& cu_q, const Tensor& positions, const Tensor& slots, int H, int G, int d, int dv);
   // width: the row length of the result (at least H * dv; the columns beyond are zero).
   Tensor delta_out(const Tensor& o, const Tensor& gate, const Tensor& w, int H, int dv, float eps, int64_t width);
+  // ---- a stream whose embedding is scaled, sums of branches, the mean of two normed branches (stream.hip)
+  Tensor embed_scaled(const Tensor& table, const Tensor& ids, float scale);
+  // stream += a + b (b may be null); a and b floats or elements of the stream's shape.
+  void stream_add(Tensor& stream, const Tensor& a, const Tensor* b);
+  // ca * norm(a) * wa + cb * norm(b) * wb as floats; a, b elements [T, H].
+  Tensor stream_pair_norm(const Tensor& a, const Tensor& wa, const Tensor& b, const Tensor& wb, float eps, float ca, float cb);
+  // qkv_post whose rotation computes its angles: pair c of every q and k head turns by position * inv_freq[c] (32-bit),
+  // cosine and sine times mag; no head norms.
+  Tensor qkv_post_angles(const Tensor& qkv, int nq, int nkv, int d, const Tensor* k_cache, const Tensor* v_cache, int page_size,
+                         const Tensor& inv_freq, float mag, const Tensor& positions, const Tensor* slots);
+  // ---- a state-space recurrence with one decay per head (ssm.hip)
+  // xbc: floats [T, C] with x (H heads of P) from column 0, B (G groups of N) from b_col, C from c_col; dt: head h's step
+  // size before its activation at column dt_col + h of proj (elements).  Returns y [T, H, P] floats; the state moves on.
+  Tensor ssm_scan(const Tensor& xbc, int64_t b_col, int64_t c_col, const Tensor& proj, int64_t dt_col, const Tensor& dt_bias, const Tensor& A_log,
+                  const Tensor& D, Tensor& state, const Tensor& cu_q, const Tensor& positions, const Tensor& slots, int H, int G, int N, int P);
+  // (y * silu(z)) normed in `parts` equal parts, times w, as elements [T, width] (columns beyond y's are zero); z: the
+  // columns [z_col, z_col + inner) of proj.
+  Tensor ssm_gate_norm(const Tensor& y, const Tensor& proj, int64_t z_col, const Tensor& w, int parts, float eps, int64_t width);
+  // ---- a mixture of experts (moe.hip)
+  struct MoePlan {
+    Tensor idx, wts;                            // [T, top]
+    Tensor row_pair, pair_row, tile_expert;
+    int top = 0, experts = 0;
+  };
+  MoePlan moe_route(const Tensor& h, const Tensor& router, int top, float weight_eps);
+  // relu(h W_up^T)^2 of every (token, choice) in the plan's rows; w_up [E, ff, width]; result [rows, ff] elements.
+  Tensor moe_up(const Tensor& h, const Tensor& w_up, const MoePlan& plan);
+  // The weighted sum of the chosen experts' down projections, floats [T, width]; w_down [E, width, ff].
+  Tensor moe_down_sum(const Tensor& act, const Tensor& w_down, const MoePlan& plan, int64_t T);
   int segment_keys() const { return segment_keys_; }
   int item_rows() const { return item_rows_; }
 

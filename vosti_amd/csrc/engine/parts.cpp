@@ -32,9 +32,13 @@ bool block_registered(const std::string& kind) { return block_registry().count(k
 namespace {
 std::string missing_in(const std::string& category, const PartSpec& p) {
   if (!part_registered(category, p.kind)) return category + " part '" + p.kind + "'";
-  // Parts below a part: the name says the category ("q_norm", "k_norm": norms; "position").
+  // Parts below a part: the name says the category ("q_norm", "k_norm": norms; "position"; "left_mixer": a mixer).
+  auto ends_with = [](const std::string& s, const char* tail) {
+    const size_t n = std::char_traits<char>::length(tail);
+    return s.size() >= n && s.compare(s.size() - n, n, tail) == 0;
+  };
   for (const auto& c : p.parts) {
-    const std::string below = c.first == "position" ? "position" : (c.first.size() >= 4 && c.first.compare(c.first.size() - 4, 4, "norm") == 0 ? "norm" : "");
+    const std::string below = c.first == "position" ? "position" : (ends_with(c.first, "norm") ? "norm" : (ends_with(c.first, "mixer") ? "mixer" : ""));
     if (below.empty()) continue;
     const std::string m = missing_in(below, *c.second);
     if (!m.empty()) return m;
@@ -74,11 +78,12 @@ void load_plugin(const std::string& path) {
 }
 
 std::pair<Tensor, Tensor> PositionEncoding::apply(const Tensor& q, const Tensor& k, const Tensor& positions) {
-  const Tensor *cos = cos_table(), *sin = sin_table();
-  if (!cos || !sin) throw EngineError("a position encoding needs tables of angles or an apply() of its own");
+  const Tensor *cos = cos_table(), *sin = sin_table(), *freq = angle_frequencies();
+  if ((!cos || !sin) && !freq) throw EngineError("a position encoding needs tables of angles, frequencies or an apply() of its own");
   auto rotate = [&](const Tensor& x) {
     if (x.shape.size() != 3) throw EngineError("position encoding of " + x.describe() + ", expected [tokens, heads, head size]");
     const int64_t T = x.dim(0), n = x.dim(1), d = x.dim(2);
+    if (freq) return kernels.qkv_post_angles(x.view({T, n * d}), (int)n, 0, (int)d, nullptr, nullptr, 0, *freq, magnitude(), positions, nullptr);
     return kernels.qkv_post(x.view({T, n * d}), (int)n, 0, (int)d, nullptr, nullptr, 0, nullptr, nullptr, 0.f, cos, sin, &positions, nullptr);
   };
   return {rotate(q), k.data ? rotate(k) : Tensor()};
@@ -225,6 +230,21 @@ class SinusoidEmbedding : public Embedding {
   Tensor weight_, inv_freq_;
 };
 
+// h[t] = E[ids[t]] * scale, as the residual stream in 32-bit whatever the element type.
+class ScaledEmbedding : public Embedding {
+ public:
+  ScaledEmbedding(const PartSpec& s, Kernels& k)
+      : Embedding(k), vocab_(s.integer("vocab_size")), hidden_(s.integer("hidden_size")), scale_((float)s.number("scale", 1.0)) {}
+  std::vector<ParamDecl> params() const override { return {{"weight", {vocab_, hidden_}}}; }
+  void load(std::map<std::string, Tensor>& t) override { weight_ = need(t, "weight"); }
+  Tensor forward(const Tensor& ids) override { return kernels.embed_scaled(weight_, ids, scale_); }
+
+ private:
+  int64_t vocab_, hidden_;
+  float scale_;
+  Tensor weight_;
+};
+
 // y = (x * rsqrt(mean(x^2) + eps)) * w in 32-bit (kernels/triton_kernels/rmsnorm.py:63-93); with a residual
 // the norm sees the unrounded sum (kernels/triton_kernels/rmsnorm_residual.py:73-125).
 class RMSNorm : public Norm {
@@ -311,6 +331,29 @@ class Rotary : public PositionEncoding {
   std::shared_ptr<Tables> tables_;
 };
 
+// The same half-rotation with angles that are computed where they are used, in 32-bit, and frequencies whose long
+// wavelengths are stretched (rotary_stretched_frequencies has the rule): numbers rotary_dim, theta and, for a stretch,
+// factor, original, fast, slow.  Cosine and sine are multiplied by 0.1 ln(factor) + 1.
+class RotaryStretched : public PositionEncoding {
+ public:
+  RotaryStretched(const PartSpec& s, Kernels& k) : PositionEncoding(k), head_dim_(s.integer("head_dim")), rotary_dim_(s.integer("rotary_dim")) {
+    if (rotary_dim_ % 2 || rotary_dim_ <= 0 || rotary_dim_ > head_dim_)
+      throw ConfigError("rotary width " + std::to_string(rotary_dim_) + " must be even and at most the head size " + std::to_string(head_dim_));
+    std::vector<float> f((size_t)rotary_dim_ / 2);
+    mag_ = rotary_stretched_frequencies(s.number("theta"), (int)rotary_dim_, s.number("factor", 0.0), s.number("original", 1.0), s.number("fast", 1.0),
+                                        s.number("slow", 1.0), f.data());
+    freq_ = zero_weight({rotary_dim_ / 2}, DType::F32);
+    hip_check(hipMemcpy(freq_.data, f.data(), f.size() * sizeof(float), hipMemcpyHostToDevice), "rotation frequencies");
+  }
+  const Tensor* angle_frequencies() override { return &freq_; }
+  float magnitude() override { return mag_; }
+
+ private:
+  int64_t head_dim_, rotary_dim_;
+  float mag_ = 1.f;
+  Tensor freq_;
+};
+
 // The attention kernels work on items: a single decoded token, or up to item_rows() consecutive rows of a
 // sequence that brings several tokens.  The item lists are the same for every attention layer of a step.
 struct AttentionItems {
@@ -328,7 +371,9 @@ struct AttentionItems {
 // and v projections with biases), softcap (score <- softcap * tanh(score / softcap)), keep_first (with a window: the
 // first keys of a sequence stay visible), sink (a learned number per head whose exponential joins the softmax's
 // denominator), exact_weights (the probabilities meet the values in 32-bit), own_kv 0 (the layer has no key and
-// value projections: it always reads another execution's cache).  The cache and the kernels see one head size: the
+// value projections: it always reads another execution's cache), block (positions are cut into blocks of this many from
+// the sequence's start, and a query sees the earlier keys of its own block only; sink 2 is the constant 0 as every
+// head's sink).  The cache and the kernels see one head size: the
 // larger of the two, rounded up to 16; the shorter of keys and values is padded with zeros in the weights, so that
 // the projections write the padding and the output projection ignores it.
 class Attention : public Mixer {
@@ -337,21 +382,23 @@ class Attention : public Mixer {
       : Mixer(k), hidden_(s.integer("hidden_size")), nq_((int)s.integer("num_heads")), nkv_((int)s.integer("num_kv_heads")),
         dk_((int)s.integer("head_dim")), dv_((int)s.integer("value_dim", s.integer("head_dim"))), scale_((float)s.number("scale")),
         window_((int)s.integer("window", 0)), keep_((int)s.integer("keep_first", 0)), softcap_((float)s.number("softcap", 0.0)),
-        bias_(s.integer("bias", 0) != 0), sink_(s.integer("sink", 0) != 0), exact_(s.integer("exact_weights", 0) != 0),
-        own_kv_(s.integer("own_kv", 1) != 0) {
+        bias_(s.integer("bias", 0) != 0), sink_((int)s.integer("sink", 0)), exact_(s.integer("exact_weights", 0) != 0),
+        own_kv_(s.integer("own_kv", 1) != 0), block_((int)s.integer("block", 0)) {
     d_ = (int)round_up(std::max(dk_, dv_), 16);
     if (nq_ % nkv_) throw ConfigError(std::to_string(nq_) + " heads are not a multiple of " + std::to_string(nkv_) + " kv heads");
     if (dk_ < 1 || dv_ < 1 || d_ > 256)
       throw ConfigError("head sizes " + std::to_string(dk_) + " and " + std::to_string(dv_) + ": the attention kernels take up to 256");
     if (window_ == 0) keep_ = 0;
+    if (block_ < 0 || (block_ > 0 && window_ > 0)) throw ConfigError("attention: blocks of positions and a window exclude each other");
+    if (sink_ < 0 || sink_ > 2) throw ConfigError("attention: 'sink' is 0 (none), 1 (a learned number per head) or 2 (the constant 0)");
     if (const PartSpec* p = s.part("q_norm")) q_norm_ = build_part<Norm>("norm", *p, k);
     if (const PartSpec* p = s.part("k_norm")) k_norm_ = build_part<Norm>("norm", *p, k);
     if (const PartSpec* p = s.part("position")) position_ = build_part<PositionEncoding>("position", *p, k);
-    if ((bias_ || d_ != dk_) && (q_norm_ || k_norm_ || position_))
-      throw ConfigError("attention: biases and padded head sizes are not built together with head norms or a position encoding");
+    if ((bias_ && (q_norm_ || k_norm_ || position_)) || (d_ != dk_ && (q_norm_ || k_norm_)))
+      throw ConfigError("attention: biases are not built together with head norms or a position encoding, nor padded head sizes with head norms");
   }
   // The kernel with capped scores serves every one of these.
-  bool capped() const { return softcap_ > 0.f || keep_ > 0 || sink_ || exact_; }
+  bool capped() const { return softcap_ > 0.f || keep_ > 0 || sink_ || exact_ || block_ > 0; }
   std::vector<ParamDecl> params() const override {
     std::vector<ParamDecl> p = {{"q_proj.weight", {(int64_t)nq_ * dk_, hidden_}}, {"o_proj.weight", {hidden_, (int64_t)nq_ * dv_}}};
     if (own_kv_) {
@@ -365,7 +412,7 @@ class Attention : public Mixer {
         p.push_back({"v_proj.bias", {(int64_t)nkv_ * dv_}});
       }
     }
-    if (sink_) {
+    if (sink_ == 1) {
       ParamDecl sinks{"sinks", {(int64_t)nq_}, true, true, -1.0, 1.0};
       p.push_back(sinks);
     }
@@ -398,7 +445,8 @@ class Attention : public Mixer {
       b_qkv_ = b.size() > 1 ? stack_rows(b) : b[0];
       b_qkv_ = b_qkv_.view({b_qkv_.numel()});
     }
-    if (sink_) sinks_ = need(t, "sinks");
+    if (sink_ == 1) sinks_ = need(t, "sinks");
+    if (sink_ == 2) sinks_ = zero_weight({(int64_t)nq_}, DType::F32);      // exp(0) = 1 joins every head's denominator
   }
   // Head norms, rotation and cache store run as one launch when the norms are weighted row scales with one eps
   // and the position encoding is a rotation by tables; any other kind runs through its own methods, step by step.
@@ -407,7 +455,7 @@ class Attention : public Mixer {
     for (Norm* n : {q_norm_.get(), k_norm_.get()})
       if (n && !n->row_scale_weight()) return false;
     if (q_norm_ && k_norm_ && q_norm_->eps() != k_norm_->eps()) return false;
-    return !position_ || position_->cos_table() != nullptr;
+    return !position_ || position_->cos_table() != nullptr || position_->angle_frequencies() != nullptr;
   }
   CacheNeed cache_need() const override {
     CacheNeed n;
@@ -483,7 +531,10 @@ class Attention : public Mixer {
     if (bias_) {
       const int64_t bw = (int64_t)(nq_ + (cache.writable ? 2 * nkv_ : 0)) * d_;
       q = k.qkv_post_bias(qkv, nq_, cache.writable ? nkv_ : 0, d_, &cache.k, &cache.v, cache.page_size, &tables.slots, b_qkv_.rows(0, bw));
-    } else if (fused()) {
+    } else if (position_ && position_->angle_frequencies() && !q_norm_ && !k_norm_) {
+      q = k.qkv_post_angles(qkv, nq_, cache.writable ? nkv_ : 0, d_, &cache.k, &cache.v, cache.page_size, *position_->angle_frequencies(),
+                            position_->magnitude(), ctx.positions, &tables.slots);
+    } else if (fused() && !(position_ && position_->angle_frequencies())) {
       const Norm* en = q_norm_ ? q_norm_.get() : k_norm_.get();
       q = k.qkv_post(qkv, nq_, cache.writable ? nkv_ : 0, d_, &cache.k, &cache.v, cache.page_size,
                      q_norm_ ? q_norm_->row_scale_weight() : nullptr, k_norm_ ? k_norm_->row_scale_weight() : nullptr,
@@ -500,7 +551,7 @@ class Attention : public Mixer {
     if (prefill_items.dim(0)) {
       if (capped())
         k.paged_attention_capped(out, q, cache.k, cache.v, tables.block_table, ctx.cu_q, ctx.k_len, prefill_items, 0, scale_, window_, keep_,
-                                 softcap_, sinks, ctx.host->k_len_bound, 0, nullptr);
+                                 softcap_, sinks, ctx.host->k_len_bound, 0, nullptr, block_);
       else
         k.paged_attention(out, q, cache.k, cache.v, tables.block_table, ctx.cu_q, ctx.k_len, prefill_items, 0, scale_, window_,
                           ctx.host->k_len_bound, 0, nullptr);
@@ -509,7 +560,7 @@ class Attention : public Mixer {
       const Tensor scratch = ctx.workspace(k.attn_scratch_floats((int)decode_items.dim(0), nq_, d_, m.nseg));
       if (capped())
         k.paged_attention_capped(out, q, cache.k, cache.v, tables.block_table, ctx.cu_q, ctx.k_len, decode_items, 1, scale_, window_, keep_,
-                                 softcap_, sinks, m.decode_bound, m.nseg, &scratch);
+                                 softcap_, sinks, m.decode_bound, m.nseg, &scratch, block_);
       else
         k.paged_attention(out, q, cache.k, cache.v, tables.block_table, ctx.cu_q, ctx.k_len, decode_items, 1, scale_, window_,
                           m.decode_bound, m.nseg, &scratch);
@@ -543,7 +594,10 @@ class Attention : public Mixer {
   float scale_;
   int window_, keep_;
   float softcap_;
-  bool bias_, sink_, exact_, own_kv_;
+  bool bias_;
+  int sink_;                          // 0: none, 1: a learned number per head, 2: the constant 0
+  bool exact_, own_kv_;
+  int block_;                         // > 0: a row sees the keys of its own block of this many positions only
   std::unique_ptr<Norm> q_norm_, k_norm_;
   std::unique_ptr<PositionEncoding> position_;
   Tensor w_qkv_, w_o_, b_qkv_, sinks_;
@@ -643,6 +697,14 @@ class LinearHead : public Head {
   Tensor weight_;
 };
 
+// Which sequence of the step every token belongs to: what a short convolution over a step's rows needs.
+void token_sequences(HostStep& step, std::vector<std::pair<std::string, HostArray>>& out) {
+  HostArray a;
+  for (size_t s = 0; s < step.q_lens.size(); ++s) a.data.insert(a.data.end(), (size_t)step.q_lens[s], (int32_t)s);
+  a.shape = {(int64_t)a.data.size()};
+  out.emplace_back("delta.token_seq", std::move(a));
+}
+
 // The gated delta rule with one decay per head and key channel.  For the mixer's input h:
 //   q = W_q h, k = W_k h (kv heads x key size), v = W_v h (heads x value size), each through a short causal
 //   convolution per channel (taps [channels, K], the last tap the current token's, zeros before a sequence's start)
@@ -717,12 +779,7 @@ class ChannelDelta : public Mixer {
   }
   // Which sequence of the step every token belongs to.
   const char* step_inputs_key() const override { return "delta.token_seq"; }
-  void step_inputs(HostStep& step, std::vector<std::pair<std::string, HostArray>>& out) override {
-    HostArray a;
-    for (size_t s = 0; s < step.q_lens.size(); ++s) a.data.insert(a.data.end(), (size_t)step.q_lens[s], (int32_t)s);
-    a.shape = {(int64_t)a.data.size()};
-    out.emplace_back("delta.token_seq", std::move(a));
-  }
+  void step_inputs(HostStep& step, std::vector<std::pair<std::string, HostArray>>& out) override { token_sequences(step, out); }
 
   Tensor forward(const Tensor& x, StepContext& ctx, CacheEntry& cache) override {
     if (cache.kind != CacheNeed::State) throw EngineError("the delta rule was handed a cache entry without state");
@@ -827,6 +884,221 @@ class SandwichDepthBlock : public Block {
   Tensor weights_;
 };
 
+// A state-space recurrence with one decay per head.  For the mixer's input h, with inner = heads * value size P, the
+// state size N and G groups:  W_in h = [z: inner | x: inner | B: G N | C: G N | dt: heads];  x, B and C together pass a
+// short causal convolution per channel (taps [channels, K] with the last tap the current token's, a bias, zeros before a
+// sequence's start) and silu;  dt <- softplus(dt + dt_bias);  per head (its B and C are those of group head / (heads /
+// G)), token by token:  S <- exp(-exp(A_log) dt) S + dt B x^T  (S is N x P),  y = S^T C + D x;  the heads' y side by
+// side times silu(z), divided in `norm_groups` equal parts each by its own root mean square, times a weight; then W_o.
+// A request's state slot holds the heads' S in 32-bit and the convolution's last K - 1 inputs.  Everything between the
+// two projections is 32-bit (ssm.hip and the convolution of delta.hip).
+class StateSpace : public Mixer {
+ public:
+  StateSpace(const PartSpec& s, Kernels& k)
+      : Mixer(k), hidden_(s.integer("hidden_size")), H_((int)s.integer("num_heads")), P_((int)s.integer("value_dim")),
+        N_((int)s.integer("state_dim")), G_((int)s.integer("groups")), parts_((int)s.integer("norm_groups", 1)),
+        taps_((int)s.integer("conv_taps")), eps_((float)s.number("eps")) {
+    if (H_ % G_) throw ConfigError(std::to_string(H_) + " heads are not a multiple of " + std::to_string(G_) + " groups");
+    if (taps_ < 1 || taps_ > 17) throw ConfigError("a short convolution of " + std::to_string(taps_) + " taps: 1 to 17 are built");
+    if (N_ > 256) throw ConfigError("a state of " + std::to_string(N_) + " rows a head: up to 256 are built");
+    inner_ = (int64_t)H_ * P_;
+    if (parts_ < 1 || inner_ % parts_) throw ConfigError(std::to_string(parts_) + " norm groups do not divide " + std::to_string(inner_) + " channels");
+    channels_ = inner_ + 2 * (int64_t)G_ * N_;
+  }
+  std::vector<ParamDecl> params() const override {
+    auto uniform = [](const char* name, std::vector<int64_t> shape, double lo, double hi) {
+      ParamDecl p{name, std::move(shape), true, true, lo, hi};
+      return p;
+    };
+    ParamDecl in{"in_proj.weight", {inner_ + channels_ + H_, hidden_}}, taps{"conv.weight", {channels_, taps_}};
+    in.p0 = 0.05;
+    taps.p0 = 0.3;
+    return {in, taps, uniform("conv.bias", {channels_}, -0.1, 0.1), uniform("dt_bias", {(int64_t)H_}, -2.0, 0.0), uniform("A_log", {(int64_t)H_}, -1.0, 1.0),
+            uniform("D", {(int64_t)H_}, 0.5, 1.5), uniform("out_norm.weight", {inner_}, 0.9, 1.1), {"o_proj.weight", {hidden_, inner_}}};
+  }
+  void load(std::map<std::string, Tensor>& t) override {
+    w_in_ = need(t, "in_proj.weight");
+    conv_ = need(t, "conv.weight");
+    conv_bias_ = need(t, "conv.bias");
+    if (conv_bias_.dtype != kernels.dtype()) throw EngineError("the convolution's bias must have the element type");
+    dt_bias_ = need(t, "dt_bias");
+    A_log_ = need(t, "A_log");
+    D_ = need(t, "D");
+    out_norm_ = need(t, "out_norm.weight");
+    inner_run_ = round_up(inner_, 8);                              // the read-out's width as whole 16-byte vectors
+    w_o_ = pad_matrix(need(t, "o_proj.weight"), hidden_, inner_run_);
+  }
+  CacheNeed cache_need() const override {
+    CacheNeed n;
+    n.kind = CacheNeed::State;
+    n.state_shape = {state_floats() + (int64_t)(taps_ - 1) * channels_};
+    n.state_dtype = DType::F32;
+    return n;
+  }
+  const char* step_inputs_key() const override { return "delta.token_seq"; }
+  void step_inputs(HostStep& step, std::vector<std::pair<std::string, HostArray>>& out) override { token_sequences(step, out); }
+
+  Tensor forward(const Tensor& x, StepContext& ctx, CacheEntry& cache) override {
+    if (cache.kind != CacheNeed::State) throw EngineError("the state-space mixer was handed a cache entry without state");
+    Kernels& k = kernels;
+    const Tensor proj = k.gemm(x, w_in_);
+    const Tensor xbc = k.delta_conv(proj, conv_, cache.state, state_floats(), ctx.inputs.at("delta.token_seq"), ctx.cu_q, ctx.positions,
+                                    ctx.state_slots, inner_, &conv_bias_);
+    const Tensor y = k.ssm_scan(xbc, inner_, inner_ + (int64_t)G_ * N_, proj, inner_ + channels_, dt_bias_, A_log_, D_, cache.state, ctx.cu_q,
+                                ctx.positions, ctx.state_slots, H_, G_, N_, P_);
+    return k.gemm(k.ssm_gate_norm(y, proj, 0, out_norm_, parts_, eps_, inner_run_), w_o_);
+  }
+
+ private:
+  int64_t state_floats() const { return (int64_t)H_ * P_ * N_; }
+  int64_t hidden_;
+  int H_, P_, N_, G_, parts_, taps_;
+  float eps_;
+  int64_t inner_ = 0, channels_ = 0, inner_run_ = 0;
+  Tensor w_in_, conv_, conv_bias_, dt_bias_, A_log_, D_, out_norm_, w_o_;
+};
+
+// Two mixers side by side that read the same input: out = (norm(left(h)) * w_left + norm(right(h)) * w_right) / 2, each
+// output divided by its root mean square over the width, in 32-bit.  One of them may keep pages and the other a state:
+// the pair asks for both, and each half gets its own.
+class PairMean : public Mixer {
+ public:
+  PairMean(const PartSpec& s, Kernels& k) : Mixer(k), hidden_(s.integer("hidden_size")), eps_((float)s.number("eps")) {
+    const PartSpec *l = s.part("left_mixer"), *r = s.part("right_mixer");
+    if (!l || !r) throw ConfigError("a pair of mixers needs the parts 'left_mixer' and 'right_mixer'");
+    left_ = build_part<Mixer>("mixer", *l, k);
+    right_ = build_part<Mixer>("mixer", *r, k);
+    const CacheNeed a = left_->cache_need(), b = right_->cache_need();
+    if ((a.kind == CacheNeed::Pages && b.kind == CacheNeed::Pages) || (a.kind == CacheNeed::State && b.kind == CacheNeed::State))
+      throw ConfigError("a pair of mixers that both keep pages, or both a state, is not built");
+  }
+  std::vector<ParamDecl> params() const override {
+    ParamDecl l{"left_out", {hidden_}, true, true, 0.9, 1.1}, r{"right_out", {hidden_}, true, true, 0.9, 1.1};
+    return {l, r};
+  }
+  std::vector<std::pair<std::string, Part*>> children() override { return {{"left", left_.get()}, {"right", right_.get()}}; }
+  void load(std::map<std::string, Tensor>& t) override {
+    w_left_ = need(t, "left_out");
+    w_right_ = need(t, "right_out");
+  }
+  CacheNeed cache_need() const override {
+    const CacheNeed a = left_->cache_need(), b = right_->cache_need();
+    CacheNeed n = a.kind == CacheNeed::Pages ? a : (b.kind == CacheNeed::Pages ? b : (a.kind == CacheNeed::State ? a : b));
+    const CacheNeed& other = a.kind == CacheNeed::State ? a : b;
+    if (n.kind == CacheNeed::Pages && other.kind == CacheNeed::State) {
+      n.state_shape = other.state_shape;
+      n.state_dtype = other.state_dtype;
+    }
+    return n;
+  }
+  Tensor forward(const Tensor& x, StepContext& ctx, CacheEntry& cache) override {
+    const Tensor l = half(*left_, x, ctx, cache), r = half(*right_, x, ctx, cache);
+    return kernels.stream_pair_norm(l, w_left_, r, w_right_, eps_, 0.5f, 0.5f);
+  }
+
+ private:
+  // A half sees the entry as the kind it asked for.
+  Tensor half(Mixer& m, const Tensor& x, StepContext& ctx, CacheEntry& cache) {
+    const CacheNeed::Kind kind = m.cache_need().kind;
+    if (kind == cache.kind) return m.forward(x, ctx, cache);
+    CacheEntry own = cache;
+    own.kind = kind;
+    if (kind == CacheNeed::State && !own.state.data) throw EngineError("a pair of mixers was handed a cache entry without the state of one half");
+    return m.forward(x, ctx, own);
+  }
+  int64_t hidden_;
+  float eps_;
+  std::unique_ptr<Mixer> left_, right_;
+  Tensor w_left_, w_right_;
+};
+
+// A mixture of `experts` small feed-forward layers without biases, W_down max(W_up h, 0)^2, of which every token uses
+// `top`: router logits W_router h in 32-bit, a softmax over all experts, the `top` largest scores, divided by their
+// sum plus weight_eps; the output is the weighted sum of the chosen experts' outputs, in 32-bit.  The experts' weights
+// lie stacked, [experts, ff, width] and [experts, width, ff] (ff padded to whole 16-byte vectors with zeros), and the
+// two projections run as grouped products over the (token, choice) pairs sorted by expert (moe.hip).
+class RoutedExperts : public FeedForward {
+ public:
+  RoutedExperts(const PartSpec& s, Kernels& k)
+      : FeedForward(k), hidden_(s.integer("hidden_size")), inter_(s.integer("intermediate_size")), experts_((int)s.integer("experts")),
+        top_((int)s.integer("top")), weight_eps_((float)s.number("weight_eps", 0.0)) {
+    if (experts_ < 1 || top_ < 1 || top_ > experts_) throw ConfigError("a mixture of " + std::to_string(experts_) + " experts cannot choose " + std::to_string(top_));
+  }
+  std::vector<ParamDecl> params() const override {
+    std::vector<ParamDecl> p = {{"router.weight", {(int64_t)experts_, hidden_}}};
+    p[0].p0 = 0.1;
+    for (int e = 0; e < experts_; ++e) {
+      p.push_back({"experts." + std::to_string(e) + ".up_proj.weight", {inter_, hidden_}});
+      p.push_back({"experts." + std::to_string(e) + ".down_proj.weight", {hidden_, inter_}});
+    }
+    return p;
+  }
+  void load(std::map<std::string, Tensor>& t) override {
+    router_ = need(t, "router.weight");
+    const int64_t padded = round_up(inter_, 8);
+    std::vector<Tensor> up, down;
+    for (int e = 0; e < experts_; ++e) {
+      up.push_back(pad_matrix(need(t, "experts." + std::to_string(e) + ".up_proj.weight"), padded, hidden_));
+      Tensor d = pad_matrix(need(t, "experts." + std::to_string(e) + ".down_proj.weight"), hidden_, padded);
+      down.push_back(d.view({hidden_ * padded / 8, 8}));     // stacked as rows of one width whatever the matrices' own
+    }
+    w_up_ = stack_rows(up).view({(int64_t)experts_, padded, hidden_});
+    w_down_ = stack_rows(down).view({(int64_t)experts_, hidden_, padded});
+  }
+  Tensor forward(const Tensor& x, StepContext&) override {
+    const Kernels::MoePlan plan = kernels.moe_route(x, router_, top_, weight_eps_);
+    return kernels.moe_down_sum(kernels.moe_up(x, w_up_, plan), w_down_, plan, x.dim(0));
+  }
+
+ private:
+  int64_t hidden_, inter_;
+  int experts_, top_;
+  float weight_eps_;
+  Tensor router_, w_up_, w_down_;
+};
+
+// Mixer and feed-forward side by side on a residual stream x in 32-bit: x <- x + (mixer(norm_mixer_in(x)) +
+// ffn(norm_ffn_in(x))), both norms of the same x; without a feed-forward, x <- x + mixer(norm_mixer_in(x)).
+class ParallelSumBlock : public Block {
+ public:
+  ParallelSumBlock(Kernels& k, std::unique_ptr<Mixer> mixer, std::unique_ptr<FeedForward> ffn, std::map<std::string, std::unique_ptr<Norm>> norms,
+                   const std::map<std::string, double>& numbers)
+      : Block(k), mixer_(std::move(mixer)), ffn_(std::move(ffn)), norms_(std::move(norms)) {
+    auto it = numbers.find("hidden_size");
+    if (it == numbers.end()) throw ConfigError("a parallel_sum block needs the number 'hidden_size'");
+    hidden_ = (int64_t)it->second;
+    has_ffn_ = dynamic_cast<NoFeedForward*>(ffn_.get()) == nullptr;
+    if (!norms_.count("mixer_in")) throw ConfigError("a parallel_sum block needs the norm 'mixer_in'");
+    if (has_ffn_ && !norms_.count("ffn_in")) throw ConfigError("a parallel_sum block with a feed-forward needs the norm 'ffn_in'");
+  }
+  std::vector<std::pair<std::string, Part*>> children() override {
+    std::vector<std::pair<std::string, Part*>> c = {{"mixer", mixer_.get()}, {"feed_forward", ffn_.get()}};
+    for (auto& n : norms_) c.emplace_back("norms." + n.first, n.second.get());
+    return c;
+  }
+  Mixer& mixer() override { return *mixer_; }
+  std::pair<Tensor, Tensor> forward(const Tensor& hidden, Tensor residual, StepContext& ctx, CacheEntry& cache) override {
+    if (hidden.dtype != DType::F32 || hidden.shape.size() != 2 || hidden.dim(1) != hidden_)
+      throw EngineError("a parallel_sum block takes the 32-bit residual stream, not " + hidden.describe());
+    Tensor stream = hidden;
+    const Tensor mixed = mixer_->forward(norms_["mixer_in"]->forward(hidden), ctx, cache);
+    if (has_ffn_) {
+      const Tensor fed = ffn_->forward(norms_["ffn_in"]->forward(hidden), ctx);
+      kernels.stream_add(stream, mixed, &fed);
+    } else {
+      kernels.stream_add(stream, mixed, nullptr);
+    }
+    return {stream, residual};
+  }
+
+ private:
+  std::unique_ptr<Mixer> mixer_;
+  std::unique_ptr<FeedForward> ffn_;
+  std::map<std::string, std::unique_ptr<Norm>> norms_;
+  int64_t hidden_ = 0;
+  bool has_ffn_ = true;
+};
+
 template <class T>
 PartFactory factory() {
   return [](const PartSpec& s, Kernels& k) { return std::unique_ptr<Part>(new T(s, k)); };
@@ -844,6 +1116,15 @@ void register_standard_parts() {
     register_block("sandwich_depth", [](Kernels& k, std::unique_ptr<Mixer> m, std::unique_ptr<FeedForward> f,
                                         std::map<std::string, std::unique_ptr<Norm>> n, const std::map<std::string, double>& numbers) {
       return std::unique_ptr<Block>(new SandwichDepthBlock(k, std::move(m), std::move(f), std::move(n), numbers));
+    });
+    register_part("embedding", "token_embedding_scaled", factory<ScaledEmbedding>());
+    register_part("position", "rotary_stretched", factory<RotaryStretched>());
+    register_part("mixer", "state_space", factory<StateSpace>());
+    register_part("mixer", "pair_mean", factory<PairMean>());
+    register_part("feed_forward", "routed_experts", factory<RoutedExperts>());
+    register_block("parallel_sum", [](Kernels& k, std::unique_ptr<Mixer> m, std::unique_ptr<FeedForward> f,
+                                      std::map<std::string, std::unique_ptr<Norm>> n, const std::map<std::string, double>& numbers) {
+      return std::unique_ptr<Block>(new ParallelSumBlock(k, std::move(m), std::move(f), std::move(n), numbers));
     });
     register_part("norm", "rmsnorm", factory<RMSNorm>());
     register_part("position", "rotary", factory<Rotary>());

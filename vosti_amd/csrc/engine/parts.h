@@ -63,7 +63,7 @@ struct CacheNeed {
   enum Kind { None, Pages, State } kind = None;
   int num_kv_heads = 0, head_dim = 0, window = 0;    // Pages
   int keep_first = 0;                                // Pages with a window: the first keys that stay visible and are never given back
-  std::vector<int64_t> state_shape;                  // State: per request
+  std::vector<int64_t> state_shape;                  // State: per request.  Pages with a shape here: the mixer keeps both
   DType state_dtype = DType::F32;
 };
 
@@ -122,6 +122,10 @@ class PositionEncoding : public Part {
   // A rotation by tabulated angles gives its tables [positions, half]; a mixer may then rotate inside a launch of its own.
   virtual const Tensor* cos_table() { return nullptr; }
   virtual const Tensor* sin_table() { return nullptr; }
+  // A rotation that computes its angles instead gives the pairs' frequencies [half] (32-bit; pair c of a head is its
+  // elements c and c + half, the angle position * frequency) and the factor on every cosine and sine.
+  virtual const Tensor* angle_frequencies() { return nullptr; }
+  virtual float magnitude() { return 1.f; }
   // Encodes positions [T] into q [T, heads, d] and k [T, kv heads, d]; k may have no memory (only q is wanted).
   // The default rotates by the tables above; a kind without tables brings its own.
   virtual std::pair<Tensor, Tensor> apply(const Tensor& q, const Tensor& k, const Tensor& positions);

@@ -25,7 +25,7 @@ CachePool::CachePool(DecoderModel& model, int page_size_, int num_pages, int num
   for (const CacheNeed& n : needs) {
     const std::pair<int, int> kind{n.window, n.window ? n.keep_first : 0};
     if (n.kind == CacheNeed::Pages && std::find(kinds.begin(), kinds.end(), kind) == kinds.end()) kinds.push_back(kind);
-    if (n.kind == CacheNeed::State) has_state = true;
+    if (n.kind == CacheNeed::State || (n.kind == CacheNeed::Pages && !n.state_shape.empty())) has_state = true;
   }
   std::sort(kinds.begin(), kinds.end());                     // 0 (all keys) first
   if (kinds.empty()) kinds.push_back({0, 0});
@@ -55,6 +55,12 @@ CachePool::CachePool(DecoderModel& model, int page_size_, int num_pages, int num
       e.k = zeroed({num_pages, n.num_kv_heads, page_size, n.head_dim}, dtype);
       e.v = zeroed({num_pages, n.num_kv_heads, n.head_dim, page_size}, dtype);
       bytes_ += e.k.bytes() + e.v.bytes();
+      if (!n.state_shape.empty()) {          // a mixer of two halves: pages for one, a state slot for the other
+        std::vector<int64_t> shape = {num_slots};
+        shape.insert(shape.end(), n.state_shape.begin(), n.state_shape.end());
+        e.state = zeroed(shape, n.state_dtype);
+        bytes_ += e.state.bytes();
+      }
     } else if (n.kind == CacheNeed::State) {
       e.kind = CacheNeed::State;
       std::vector<int64_t> shape = {num_slots};

@@ -13,6 +13,15 @@ namespace vosti {
 // the reciprocal is a 32-bit division.
 void rotary_inverse_frequencies(double theta, int rotary_dim, float* out);
 
+// The frequencies of a rotation whose long wavelengths are stretched by `factor` so that positions beyond `original`
+// stay inside the angles the model was trained on: with f[j] = theta^(-2j / rotary_dim) and
+// turn(t) = rotary_dim * ln(original / (2 pi t)) / (2 ln theta), the pair whose wavelength makes t turns over `original`
+// positions, lo = max(floor(turn(fast)), 0), hi = min(ceil(turn(slow)), rotary_dim - 1) and
+// ramp[j] = clamp((j - lo) / max(hi - lo, 0.001), 0, 1), out[j] = f[j] / factor * ramp[j] + f[j] * (1 - ramp[j]),
+// computed in 64-bit and rounded once.  Returns the factor on every cosine and sine, 0.1 ln(factor) + 1.
+// factor <= 0: no stretch (out[j] = f[j], returns 1).
+float rotary_stretched_frequencies(double theta, int rotary_dim, double factor, double original, double fast, double slow, float* out);
+
 // Recorded decode steps have one of 1, 2, 3, 4, 6, 8, 12, 16, 24, ... rows (a step with fewer is filled up with
 // rows that read one key and store nothing; the reference pads its graphs likewise,
 // python/vosti_kernels/graph_overlay.py:177-389), and block tables one of these numbers times eight pages, so

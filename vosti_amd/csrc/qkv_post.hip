@@ -26,11 +26,26 @@ struct QkvPostArgs {
   const elem_t* bias;     // [(nq + 2 nkv) d] or null: added to the row first (the sum rounded to the element type)
   const elem_t* cos_t;    // [max_pos, rot_half] or null
   const elem_t* sin_t;
+  const float* inv_freq;  // [rot_half] or null: instead of tables, the angle of pair c is position * inv_freq[c], in 32-bit,
+  float mag;              // and its cosine and sine are multiplied by this
   const int32_t* positions;  // [T]
   const int32_t* slots;      // [T]: page * P + offset, or -1
   int w_is_f32, nq, nkv, d, P, rot_half;
   float eps;
 };
+
+// Cosine and sine of pair c at a token: from the tables' row, or computed in 32-bit from the position and the pair's
+// frequency (the product rounded once, then the library's cosine and sine, each times the magnitude).
+__device__ __forceinline__ void pair_angle(const QkvPostArgs& a, int64_t trow, float posf, int c, float& cs, float& sn) {
+  if (a.inv_freq != nullptr) {
+    const float angle = posf * a.inv_freq[c];
+    cs = cosf(angle) * a.mag;
+    sn = sinf(angle) * a.mag;
+  } else {
+    cs = to_f32(a.cos_t[trow + c]);
+    sn = to_f32(a.sin_t[trow + c]);
+  }
+}
 
 // A workgroup has four waves and one token; wave w takes the heads first + w, first + w + 4, ... of the
 // workgroup's `per_wave` * 4 heads, so that a long step does not start a workgroup per head.
@@ -43,8 +58,10 @@ __global__ __launch_bounds__(256) void qkv_post_kernel(QkvPostArgs a, int per_wa
   // With a rotation half of 64 or 128 elements the partner of an element is held by the same lane.
   const bool in_lane = rh % 64 == 0;
   const int shift = rh / 64;
+  const bool has_rot = a.cos_t != nullptr || a.inv_freq != nullptr;
   int64_t trow = 0;
   if (a.cos_t != nullptr) trow = (int64_t)a.positions[tok] * rh;
+  const float posf = a.inv_freq != nullptr ? (float)a.positions[tok] : 0.f;
   const int slot = a.slots != nullptr ? a.slots[tok] : -1;
   for (int j = 0; j < per_wave; ++j) {
     const int hh = (blockIdx.y * per_wave + j) * 4 + wave;
@@ -71,8 +88,8 @@ __global__ __launch_bounds__(256) void qkv_post_kernel(QkvPostArgs a, int per_wa
         if (c < d) xv[i] = round_to_elem((xv[i] * rr) * load_weight(w, a.w_is_f32, c));
       }
     }
-    const bool rotate = a.cos_t != nullptr && kind != 2;
-    if (a.cos_t != nullptr && !in_lane) {
+    const bool rotate = has_rot && kind != 2;
+    if (has_rot && !in_lane) {
       if (rotate) {
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -90,17 +107,19 @@ __global__ __launch_bounds__(256) void qkv_post_kernel(QkvPostArgs a, int per_wa
       for (int i = 0; i < 4; ++i) {
         const int c = lane + 64 * i;
         if (c < rh) {
-          const float cs = to_f32(a.cos_t[trow + c]), sn = to_f32(a.sin_t[trow + c]);
+          float cs, sn;
+          pair_angle(a, trow, posf, c, cs, sn);
           const float other = in_lane ? (i + shift < 4 ? old[(i + shift) & 3] : 0.f) : y[c + rh];
           xv[i] = old[i] * cs - other * sn;
         } else if (c < 2 * rh) {
-          const float cs = to_f32(a.cos_t[trow + c - rh]), sn = to_f32(a.sin_t[trow + c - rh]);
+          float cs, sn;
+          pair_angle(a, trow, posf, c - rh, cs, sn);
           const float other = in_lane ? (i >= shift ? old[(i - shift) & 3] : 0.f) : y[c - rh];
           xv[i] = old[i] * cs + other * sn;
         }
       }
     }
-    if (a.cos_t != nullptr && !in_lane) __syncthreads();    // y is free for the next head
+    if (has_rot && !in_lane) __syncthreads();    // y is free for the next head
     if (!live) continue;
     if (kind == 0) {
       elem_t* o = a.q_out + ((int64_t)tok * a.nq + hh) * d;
@@ -221,24 +240,25 @@ extern "C" {
 static int qkv_post_launch(const elem_t* qkv, int64_t row_stride, elem_t* q_out, elem_t* kc, elem_t* vc, const void* q_w,
                            const void* k_w, int w_is_f32, const elem_t* cos_t, const elem_t* sin_t, int rot_half,
                            const int32_t* positions, const int32_t* slots, int T, int nq, int nkv, int d, int P, float eps,
-                           const elem_t* bias, hipStream_t st) {
+                           const elem_t* bias, hipStream_t st, const float* inv_freq = nullptr, float mag = 1.f) {
   VK_REQUIRE(T >= 0 && nq >= 0 && nkv >= 0 && nq + nkv > 0, "qkv_post: bad sizes T=%d nq=%d nkv=%d", T, nq, nkv);
   VK_REQUIRE(d > 0 && d <= 256, "qkv_post: head size %d must be in 1..256", d);
   VK_REQUIRE(row_stride >= (int64_t)(nq + 2 * nkv) * d, "qkv_post: row stride %lld too small", (long long)row_stride);
-  VK_REQUIRE(cos_t == nullptr || (rot_half > 0 && 2 * rot_half <= d), "qkv_post: rotary width %d does not fit head size %d",
+  VK_REQUIRE((cos_t == nullptr && inv_freq == nullptr) || (rot_half > 0 && 2 * rot_half <= d), "qkv_post: rotary width %d does not fit head size %d",
              2 * rot_half, d);
-  VK_REQUIRE(cos_t == nullptr || positions != nullptr, "qkv_post: rotation needs positions");
+  VK_REQUIRE((cos_t == nullptr && inv_freq == nullptr) || positions != nullptr, "qkv_post: rotation needs positions");
+  VK_REQUIRE(cos_t == nullptr || inv_freq == nullptr, "qkv_post: tables of angles or frequencies, not both");
   VK_REQUIRE(nkv == 0 || (slots != nullptr && kc != nullptr && vc != nullptr && P > 0), "qkv_post: store needs slots and caches");
   VK_REQUIRE(nq + 2 * nkv <= 65535, "qkv_post: too many heads");
   if (T == 0) return 0;
   QkvPostArgs a;
   a.qkv = qkv; a.row_stride = row_stride; a.q_out = q_out; a.kc = kc; a.vc = vc; a.q_w = q_w; a.k_w = k_w;
   a.cos_t = cos_t; a.sin_t = sin_t; a.positions = positions; a.slots = slots; a.w_is_f32 = w_is_f32; a.bias = bias;
-  a.nq = nq; a.nkv = nkv; a.d = d; a.P = P; a.rot_half = rot_half; a.eps = eps;
+  a.nq = nq; a.nkv = nkv; a.d = d; a.P = P; a.rot_half = rot_half; a.eps = eps; a.inv_freq = inv_freq; a.mag = mag;
   // Few tokens: four waves' worth of heads per workgroup, for many workgroups; many tokens: all heads of a token.
   const int heads = nq + 2 * nkv;
   const int lph = d / VK_VEC;          // lanes per head in the kernel with 16-byte accesses
-  const bool vec = (d == 64 || d == 128 || d == 256) && lph <= 64 && (cos_t == nullptr || 2 * rot_half == d) &&
+  const bool vec = inv_freq == nullptr && (d == 64 || d == 128 || d == 256) && lph <= 64 && (cos_t == nullptr || 2 * rot_half == d) &&
                    row_stride % VK_VEC == 0 && ((uintptr_t)qkv % 16) == 0 && (q_out == nullptr || (uintptr_t)q_out % 16 == 0) &&
                    (kc == nullptr || (uintptr_t)kc % 16 == 0) && (bias == nullptr || (uintptr_t)bias % 16 == 0) && (cos_t == nullptr || ((uintptr_t)cos_t % 16 == 0 && (uintptr_t)sin_t % 16 == 0));
   if (vec) {
@@ -272,6 +292,15 @@ int vk_qkv_post_bias(const elem_t* qkv, int64_t row_stride, elem_t* q_out, elem_
                      const elem_t* bias, hipStream_t st) {
   return qkv_post_launch(qkv, row_stride, q_out, kc, vc, q_w, k_w, w_is_f32, cos_t, sin_t, rot_half, positions, slots, T, nq, nkv, d, P, eps,
                          bias, st);
+}
+
+// The same with the angles computed instead of tabulated: pair c (elements c and c + rot_half of every q and k head)
+// turns by position * inv_freq[c], the product, the cosine and the sine in 32-bit, both times `mag`.
+int vk_qkv_post_angles(const elem_t* qkv, int64_t row_stride, elem_t* q_out, elem_t* kc, elem_t* vc, const float* inv_freq, float mag,
+                       int rot_half, const int32_t* positions, const int32_t* slots, int T, int nq, int nkv, int d, int P, hipStream_t st) {
+  VK_REQUIRE(inv_freq != nullptr, "qkv_post: the rotation's frequencies are missing");
+  return qkv_post_launch(qkv, row_stride, q_out, kc, vc, nullptr, nullptr, 0, nullptr, nullptr, rot_half, positions, slots, T, nq, nkv, d, P, 0.f,
+                         nullptr, st, inv_freq, mag);
 }
 
 }  // extern "C"

@@ -202,6 +202,47 @@ __global__ __launch_bounds__(256) void softcap_kernel(elem_t* x, float cap, int6
   if (e < n) x[e] = from_f32<elem_t>(cap * tanhf(to_f32(x[e]) / cap));
 }
 
+// out[t, :] = table[ids[t], :] * scale, as floats: the residual stream of a model whose embedding is multiplied by a constant.
+__global__ __launch_bounds__(STREAM_THREADS) void embed_scaled_kernel(float* __restrict__ out, const elem_t* __restrict__ table,
+                                                                      const int32_t* __restrict__ ids, int H, float scale) {
+  const elem_t* src = table + (int64_t)ids[blockIdx.x] * H;
+  float* dst = out + (int64_t)blockIdx.x * H;
+  for (int c = threadIdx.x; c < H; c += blockDim.x) dst[c] = to_f32(src[c]) * scale;
+}
+
+// out = base + (a + b) (b may be null: out = base + a), element by element; a and b are floats or elements.
+__global__ __launch_bounds__(256) void stream_add_kernel(float* out, const float* base, const void* __restrict__ a, int a_is_f32,
+                                                         const void* __restrict__ b, int b_is_f32, int64_t n) {
+  const int64_t e = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (e >= n) return;
+  float v = a_is_f32 ? static_cast<const float*>(a)[e] : to_f32(static_cast<const elem_t*>(a)[e]);
+  if (b != nullptr) v = v + (b_is_f32 ? static_cast<const float*>(b)[e] : to_f32(static_cast<const elem_t*>(b)[e]));
+  out[e] = base[e] + v;
+}
+
+// out = ca * norm_a(a) + cb * norm_b(b), rows of floats: each input row divided by its own root mean square and
+// multiplied by its own weight.  One workgroup per row, sums in stream_block_sum's order.
+__global__ __launch_bounds__(STREAM_THREADS) void stream_pair_norm_kernel(float* __restrict__ out, const elem_t* __restrict__ a,
+                                                                          const void* __restrict__ wa, const elem_t* __restrict__ b,
+                                                                          const void* __restrict__ wb, int w_is_f32, int H, float eps, float ca,
+                                                                          float cb) {
+  __shared__ float red_a[4], red_b[4];
+  const int64_t base = (int64_t)blockIdx.x * H;
+  float pa = 0.f, pb = 0.f;
+  for (int c = threadIdx.x; c < H; c += STREAM_THREADS) {
+    const float va = to_f32(a[base + c]), vb = to_f32(b[base + c]);
+    pa = pa + va * va;
+    pb = pb + vb * vb;
+  }
+  const float ra = rsqrtf(stream_block_sum(pa, red_a) / (float)H + eps);
+  const float rb = rsqrtf(stream_block_sum(pb, red_b) / (float)H + eps);
+  for (int c = threadIdx.x; c < H; c += STREAM_THREADS) {
+    const float na = (to_f32(a[base + c]) * ra) * load_weight(wa, w_is_f32, c);
+    const float nb = (to_f32(b[base + c]) * rb) * load_weight(wb, w_is_f32, c);
+    out[base + c] = ca * na + cb * nb;
+  }
+}
+
 extern "C" {
 
 int vk_embed_sinusoid(float* out, const elem_t* table, const int32_t* ids, const int32_t* positions, const float* inv_freq, int T,
@@ -270,6 +311,28 @@ int vk_softcap(elem_t* x, float cap, int64_t n, hipStream_t st) {
   if (n == 0) return 0;
   softcap_kernel<<<(unsigned)((n + 255) / 256), 256, 0, st>>>(x, cap, n);
   return vk_check_launch("softcap");
+}
+
+int vk_embed_scaled(float* out, const elem_t* table, const int32_t* ids, int T, int H, int V, float scale, hipStream_t st) {
+  VK_REQUIRE(T >= 0 && H > 0 && V > 0, "scaled embedding: bad sizes T=%d H=%d V=%d", T, H, V);
+  if (T == 0) return 0;
+  embed_scaled_kernel<<<T, STREAM_THREADS, 0, st>>>(out, table, ids, H, scale);
+  return vk_check_launch("scaled embedding");
+}
+
+int vk_stream_add(float* out, const float* base, const void* a, int a_is_f32, const void* b, int b_is_f32, int64_t n, hipStream_t st) {
+  VK_REQUIRE(n >= 0 && a != nullptr, "stream add: bad sizes");
+  if (n == 0) return 0;
+  stream_add_kernel<<<(unsigned)((n + 255) / 256), 256, 0, st>>>(out, base, a, a_is_f32, b, b_is_f32, n);
+  return vk_check_launch("stream add");
+}
+
+int vk_stream_pair_norm(float* out, const elem_t* a, const void* wa, const elem_t* b, const void* wb, int w_is_f32, int rows, int H, float eps,
+                        float ca, float cb, hipStream_t st) {
+  VK_REQUIRE(rows >= 0 && H > 0 && eps >= 0.f, "pair norm: bad sizes rows=%d H=%d", rows, H);
+  if (rows == 0) return 0;
+  stream_pair_norm_kernel<<<rows, STREAM_THREADS, 0, st>>>(out, a, wa, b, wb, w_is_f32, H, eps, ca, cb);
+  return vk_check_launch("pair norm");
 }
 
 }  // extern "C"

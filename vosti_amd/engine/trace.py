@@ -16,7 +16,7 @@ def build_parser() -> argparse.ArgumentParser:
     p.add_argument("--max-tokens", type=int, required=True,
                    help="most tokens live requests hold at any time, each request rounded up to a page")
     p.add_argument("--page-size", type=int, default=64, help="tokens per cache page (a power of two, default 64)")
-    p.add_argument("--max-requests", type=int, default=8, help="most requests alive at a time (state slots)")
+    p.add_argument("--max-requests", type=int, default=4, help="most requests alive at a time (state slots)")
     p.add_argument("--prefix-cache", action="store_true",
                    help="a request whose first tokens equal full pages that an earlier request left reuses those pages: "
                         "feed such a request its tokens from the first uncached one on (--prefix-report tells which)")
