@@ -92,8 +92,10 @@ def block_attention(h, w, pre, m):
         g = head // (H // G)
         s = (q[:, head] @ k[:, g].T) * m["scale"]
         see = torch.tensor([[block_visible(i, j, size) for j in range(T)] for i in range(T)])
-        e = torch.where(see, torch.exp(s), torch.zeros_like(s))
-        out[:, head] = (e / (1.0 + e.sum(-1, keepdim=True))) @ v[:, g]
+        # exp(s) / (1 + sum exp(s)), with everything divided by exp(top), top the row's largest visible score or 0
+        top = torch.where(see, s, torch.zeros_like(s)).amax(-1, keepdim=True).clamp(min=0.0)
+        e = torch.where(see, torch.exp(s - top), torch.zeros_like(s))
+        out[:, head] = (e / (torch.exp(-top) + e.sum(-1, keepdim=True))) @ v[:, g]
     return out.reshape(T, H * dv) @ w[pre + "o"].to(h.dtype).T
 
 

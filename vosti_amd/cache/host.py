@@ -65,6 +65,7 @@ def host_lib():
     sig("vh_describe_config", I, c_char_p, c_char_p, I, c_char_p, I)
     sig("vh_model_types", I, c_char_p, I)
     sig("vh_rotary_inverse_frequencies", None, c_double, I, c_void_p)
+    sig("vh_rotary_stretched_frequencies", ctypes.c_float, c_double, I, c_double, c_double, c_double, c_double, c_void_p)
     sig("vh_graph_row_bucket", I, I)
     sig("vh_graph_width_bucket", I, I)
     sig("vh_max_graphs", I)
@@ -112,6 +113,16 @@ def rotary_inverse_frequencies(theta: float, rotary_dim: int):
     out = np.empty(rotary_dim // 2, dtype=np.float32)
     host_lib().vh_rotary_inverse_frequencies(float(theta), int(rotary_dim), out.ctypes.data)
     return out
+
+
+def rotary_stretched_frequencies(theta: float, rotary_dim: int, factor: float = 0.0, original: float = 1.0, fast: float = 1.0, slow: float = 1.0):
+    """(float32 numpy array [rotary_dim / 2], factor on cosine and sine): the frequencies of a rotation whose long
+    wavelengths are stretched by ``factor`` (0: not at all), as the engine's rotary_stretched part computes them."""
+    import numpy as np
+    out = np.empty(rotary_dim // 2, dtype=np.float32)
+    mag = host_lib().vh_rotary_stretched_frequencies(float(theta), int(rotary_dim), float(factor), float(original), float(fast), float(slow),
+                                                     out.ctypes.data)
+    return out, float(mag)
 
 
 def graph_row_bucket(rows: int) -> int:

@@ -316,9 +316,23 @@ ModelRunner::Captured* ModelRunner::capture(const Key& key, Layout& lay) {
   workspace(workspace_needed(lay.host));
   cap->workspace = workspace_;
   int32_t* meta = static_cast<int32_t*>(cap->meta->data());
-  // Once outside a recording: the arena grows to what the step needs, and every kernel has run once.
+  // Once outside a recording: the arena grows to what the step needs, and every kernel has run once.  The recorded
+  // step runs when the graph is launched below, so this run must leave nothing behind: keys and values are written to
+  // the same places again, but a mixer's state would move on twice.  The states are put aside and brought back.
+  std::vector<std::pair<Tensor*, std::unique_ptr<DeviceBuffer>>> kept;
+  for (CacheEntry& e : pool_.entries) {
+    if (!e.state.data || !e.writable) continue;
+    bool seen = false;
+    for (auto& k : kept) seen = seen || k.first->data == e.state.data;
+    if (seen) continue;
+    kept.emplace_back(&e.state, std::make_unique<DeviceBuffer>(e.state.bytes()));
+    hip_check(hipMemcpyAsync(kept.back().second->data(), e.state.data, e.state.bytes(), hipMemcpyDeviceToDevice, k_.stream), "keeping a state");
+  }
   forward(lay, meta);
+  for (auto& k : kept)
+    hip_check(hipMemcpyAsync(k.first->data, k.second->data(), k.first->bytes(), hipMemcpyDeviceToDevice, k_.stream), "bringing a state back");
   hip_check(hipStreamSynchronize(k_.stream), "the step before its recording");
+  kept.clear();
   capturing_ = true;
   k_.arena.forbid_growth(true);
   hipError_t begun = hipStreamBeginCapture(k_.stream, hipStreamCaptureModeThreadLocal);

@@ -213,6 +213,9 @@ int vh_model_types(char* out, int cap) {
 }
 
 void vh_rotary_inverse_frequencies(double theta, int rotary_dim, float* out) { rotary_inverse_frequencies(theta, rotary_dim, out); }
+float vh_rotary_stretched_frequencies(double theta, int rotary_dim, double factor, double original, double fast, double slow, float* out) {
+  return rotary_stretched_frequencies(theta, rotary_dim, factor, original, fast, slow, out);
+}
 int vh_graph_row_bucket(int rows) { return graph_row_bucket(rows); }
 int vh_graph_width_bucket(int pages) { return graph_width_bucket(pages); }
 int vh_max_graphs(void) { return kMaxGraphs; }
