@@ -6,6 +6,7 @@
     python bench.py --workload mixed14b     # Qwen3-14B shape: 32 prompts of 128 to 4,096 tokens, prefill in portions beside decoding
     python bench.py --workload prefix32b    # Qwen3-32B shape: 64 requests at context 8,192 that share a 1,024-token prefix
     python bench.py --workload aligned      # the reference's aligned phases: batch 4, cached contexts 0 to 16K, 256 new tokens / 127 decode steps
+    python bench.py --workload povatar      # the Povatar design (attention beside a state-space recurrence, routed experts) at three layer sizes beside Tezinex at equal size
     python bench.py --workload tezinex      # the Tezinex design at three layer sizes beside the Qwen3 decoder at equal size: prefill and decode
 
 A step is one decode step of the engine (plan, forward, sample, commit) for a
@@ -86,9 +87,9 @@ def main() -> int:
     ap.add_argument("--no-other-shapes", action="store_true", help="skip the 14B and 32B workloads that the default record holds as points")
     ap.add_argument("--prompt-tokens", type=int, default=PROMPT_TOKENS,
                     help="context length of the decode measurement (the prefill figure is always of 2,048 tokens)")
-    ap.add_argument("--workload", default="decode8b", choices=["decode8b", "mixed14b", "prefix32b", "aligned", "tezinex"])
-    ap.add_argument("--sizes", default=",".join(["1k", "2k", "4k"]), help="which layer sizes --workload tezinex measures (1k, 2k, 4k)")
-    ap.add_argument("--only-design", default="", choices=["", "tezinex", "qwen3"], help="--workload tezinex: measure one of the two designs only")
+    ap.add_argument("--workload", default="decode8b", choices=["decode8b", "mixed14b", "prefix32b", "aligned", "tezinex", "povatar"])
+    ap.add_argument("--sizes", default=",".join(["1k", "2k", "4k"]), help="which layer sizes --workload tezinex / povatar measure (1k, 2k, 4k)")
+    ap.add_argument("--only-design", default="", choices=["", "tezinex", "qwen3", "povatar"], help="--workload tezinex / povatar: measure one of the two designs only")
     ap.add_argument("--engine", default="native", choices=["native", "python"],
                     help="which engine every figure is measured through: the native one (vosti_amd.engine.NativeEngine) or the "
                          "Python step function over the same kernels, cache manager and scheduler")
@@ -111,7 +112,7 @@ def main() -> int:
     if args.workload == "aligned":
         print(json.dumps(aligned_workload(args)), flush=True)
         return 0
-    if args.workload == "tezinex":
+    if args.workload in ("tezinex", "povatar"):
         print(json.dumps(tezinex_workload(args)), flush=True)
         return 0
     if args.workload != "decode8b":
@@ -531,9 +532,23 @@ def tezinex_config(width, heads, kv_heads, ff, layers, vocab):
             "width": width}
 
 
+def povatar_config(width, heads, kv_heads, ff, layers, vocab):
+    """Every layer: attention (heads of 128, keys of the query's own block of 1,024 positions, half of every head rotated
+    with stretched frequencies) beside a state-space recurrence as wide as the model (heads of 64, 128 state rows), and 16
+    experts of which a token uses 2, each half as wide as the dense feed-forward of the same size: a token's matrix work
+    is that of a Tezinex or Qwen3 layer of these sizes, plus the recurrence's projections."""
+    left = {"dim": 128, "vdim": 128, "heads": heads, "kv_heads": kv_heads, "mask": {"size": 1024}, "scale": 128 ** -0.5,
+            "rot": {"base": 10000.0, "dims": 64, "scaling": {"factor": 8.0, "fast": 32.0, "original": 4096, "slow": 1.0}}}
+    right = {"conv": 4, "groups": 2, "heads": width // 64, "norm_groups": 2, "state": 128, "vdim": 64}
+    mlp = {"kind": "moe", "expert": {"ff": ff // 2}, "router": {"experts": 16, "top": 2}}
+    return {"architecture": "Povatar", "embedding": {"scale": 1.0}, "norm": {"eps": 1e-5}, "vocab": vocab, "width": width,
+            "layers": [{"type": "parallel", "mixer": {"left": left, "right": right}, "mlp": mlp} for _ in range(layers)]}
+
+
 def tezinex_workload(args) -> dict:
     """Prefill of one prompt and decoding at a fixed batch for the Tezinex design at three layer sizes, each beside the
-    Qwen3 decoder with the same width, heads, feed-forward, layers and vocabulary (random weights, the native engine)."""
+    Qwen3 decoder with the same width, heads, feed-forward, layers and vocabulary (random weights, the native engine).
+    --workload povatar: the Povatar design beside Tezinex, its nearest neighbour here, in the same way."""
     import tempfile
     from vosti_amd.engine import NativeEngine
     from vosti_amd.sampling import SamplingParams
@@ -545,7 +560,9 @@ def tezinex_workload(args) -> dict:
     record = {"metric": "decode_tokens_per_s", "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
               "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
               "data": "synthetic: seeded random token prompts, seeded random weights", "sizes": {},
-              "config": {"model": "Tezinex (delta, attention, shared-key attention, delta, ...) beside Qwen3 at equal size", "layers": layers,
+              "config": {"model": "Povatar (attention beside a state-space recurrence, 16 experts of which 2) beside Tezinex at equal size"
+                         if args.workload == "povatar" else "Tezinex (delta, attention, shared-key attention, delta, ...) beside Qwen3 at equal size",
+                         "layers": layers,
                          "global_batch": batch, "seq_len": prompt_tokens, "vocab_size": vocab, "parallelism": "single GPU",
                          "graphs": bool(args.graphs)}}
 
@@ -587,21 +604,29 @@ def tezinex_workload(args) -> dict:
             return {"prefill_ms": round(prefill_s * 1e3, 3), "prefill_tokens_per_s": round(prompt_tokens / prefill_s, 1),
                     "decode_ms_per_step": round(step_s * 1e3, 4), "decode_tokens_per_s": round(batch / step_s, 1)}
 
+    # The design that is measured and the neighbour it stands beside.
+    first, second = ("povatar", "tezinex") if args.workload == "povatar" else ("tezinex", "qwen3")
+
+    def config_of(design, width, heads, kv_heads, ff):
+        if design == "povatar":
+            return povatar_config(width, heads, kv_heads, ff, layers, vocab)
+        if design == "tezinex":
+            return tezinex_config(width, heads, kv_heads, ff, layers, vocab)
+        return dict(QWEN3_8B, architectures=["Qwen3ForCausalLM"], vocab_size=vocab, hidden_size=width, intermediate_size=ff, num_hidden_layers=layers,
+                    num_attention_heads=heads, num_key_value_heads=kv_heads, tie_word_embeddings=True)
+
     for name in [n for n in args.sizes.split(",") if n]:
         width, heads, kv_heads, ff = TEZINEX_SIZES[name]
-        print(f"bench.py: tezinex: width {width}, {layers} layers", file=sys.stderr, flush=True)
+        print(f"bench.py: {args.workload}: width {width}, {layers} layers", file=sys.stderr, flush=True)
         point = {"width": width, "q_heads": heads, "kv_heads": kv_heads, "ff": ff}
-        if args.only_design != "qwen3":
-            point["tezinex"] = measure(tezinex_config(width, heads, kv_heads, ff, layers, vocab))
-        if args.only_design != "tezinex":
-            point["qwen3"] = measure(dict(QWEN3_8B, architectures=["Qwen3ForCausalLM"], vocab_size=vocab, hidden_size=width, intermediate_size=ff,
-                                          num_hidden_layers=layers, num_attention_heads=heads, num_key_value_heads=kv_heads,
-                                          tie_word_embeddings=True))
-        if "tezinex" in point and "qwen3" in point:
-            point["decode_ratio"] = round(point["tezinex"]["decode_tokens_per_s"] / point["qwen3"]["decode_tokens_per_s"], 3)
-            point["prefill_ratio"] = round(point["tezinex"]["prefill_tokens_per_s"] / point["qwen3"]["prefill_tokens_per_s"], 3)
+        for design in (first, second):
+            if not args.only_design or args.only_design == design:
+                point[design] = measure(config_of(design, width, heads, kv_heads, ff))
+        if first in point and second in point:
+            point["decode_ratio"] = round(point[first]["decode_tokens_per_s"] / point[second]["decode_tokens_per_s"], 3)
+            point["prefill_ratio"] = round(point[first]["prefill_tokens_per_s"] / point[second]["prefill_tokens_per_s"], 3)
         record["sizes"][name] = point
-        last = point.get("tezinex") or point["qwen3"]
+        last = point.get(first) or point[second]
         record["value"] = last["decode_tokens_per_s"]
         record["ms_per_step"] = last["decode_ms_per_step"]
     return record

@@ -259,7 +259,8 @@ def test_the_constant_in_the_denominator(tmp_path, dtype):
     # The plain implementation itself: the same scores through an ordinary softmax give another answer.
     h = plain.weighted_norm(plain.embed(tokens, w["embed"], 1.0, torch.float64), w["l0.norm1"].double(), cfg["norm"]["eps"])
     out = plain.block_attention(h, w, "l0.mix.left.", cfg["layers"][0]["mixer"]["left"])
-    assert out.abs().max() < 1e-6
+    ordinary = (h[:1] @ w["l0.mix.left.v"].double().T) @ w["l0.mix.left.o"].double().T      # all tokens are equal: the mean of the values is any of them
+    assert out.abs().max() < 0.01 * ordinary.abs().max()
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

@@ -123,11 +123,12 @@ struct Kernels::Fn {
   int (*ssm_scan)(P, CP, int64_t, int, int, CP, int64_t, CP, CP, CP, int, P, int64_t, CP, CP, CP, int, int, int, int, int, hipStream_t);
   int (*ssm_gate_norm)(P, int64_t, CP, CP, int64_t, CP, int, int, int, int, float, hipStream_t);
   int (*moe_max_tiles)(int, int, int);
-  int (*moe_route)(P, P, CP, CP, int, int, int, int, float, hipStream_t);
-  int (*moe_plan)(CP, P, P, P, int, int, int, hipStream_t);
-  int (*moe_up)(P, int64_t, CP, int64_t, CP, CP, CP, int, int, int, int, int, hipStream_t);
+  int (*moe_route)(P, P, P, CP, CP, int, int, int, int, float, hipStream_t);
+  int (*moe_plan)(CP, P, P, P, P, P, int, int, int, hipStream_t);
+  int (*moe_up)(P, int64_t, CP, int64_t, CP, CP, CP, CP, int, int, int, int, int, hipStream_t);
   int (*moe_down)(P, CP, int64_t, CP, CP, CP, int, int, int, int, int, hipStream_t);
   int (*moe_combine)(P, CP, CP, CP, int, int, int, hipStream_t);
+  int (*moe_relu_square)(P, int64_t, hipStream_t);
 };
 
 static constexpr int KERNEL_ABI = 16;
@@ -164,7 +165,7 @@ Kernels::Kernels(const std::string& lib_dir, const std::string& name) : name_(na
   VK(qkv_post_angles, "vk_qkv_post_angles"); VK(embed_scaled, "vk_embed_scaled"); VK(stream_add, "vk_stream_add");
   VK(stream_pair_norm, "vk_stream_pair_norm"); VK(ssm_scan, "vk_ssm_scan"); VK(ssm_gate_norm, "vk_ssm_gate_norm");
   VK(moe_max_tiles, "vk_moe_max_tiles"); VK(moe_route, "vk_moe_route"); VK(moe_plan, "vk_moe_plan"); VK(moe_up, "vk_moe_up");
-  VK(moe_down, "vk_moe_down"); VK(moe_combine, "vk_moe_combine");
+  VK(moe_down, "vk_moe_down"); VK(moe_combine, "vk_moe_combine"); VK(moe_relu_square, "vk_moe_relu_square");
 #undef VK
   segment_keys_ = fn_->attn_segment_keys();
   item_rows_ = fn_->attn_item_rows();
@@ -750,10 +751,14 @@ Kernels::MoePlan Kernels::moe_route(const Tensor& h, const Tensor& router, int t
   p.idx = empty({T, top}, DType::I32);
   p.wts = empty({T, top}, DType::F32);
   p.row_pair = empty({tiles * 16}, DType::I32);
+  p.row_token = empty({tiles * 16}, DType::I32);
   p.pair_row = empty({T * top}, DType::I32);
   p.tile_expert = empty({tiles}, DType::I32);
-  call(fn_->moe_route(p.idx.data, p.wts.data, h.data, router.data, (int)T, (int)h.dim(1), (int)E, top, weight_eps, stream));
-  call(fn_->moe_plan(p.idx.data, p.row_pair.data, p.pair_row.data, p.tile_expert.data, (int)T, top, (int)E, stream));
+  p.expert_start = empty({E + 1}, DType::I32);
+  Tensor logits = empty({T, E}, DType::F32);
+  call(fn_->moe_route(p.idx.data, p.wts.data, logits.data, h.data, router.data, (int)T, (int)h.dim(1), (int)E, top, weight_eps, stream));
+  call(fn_->moe_plan(p.idx.data, p.row_pair.data, p.row_token.data, p.pair_row.data, p.tile_expert.data, p.expert_start.data, (int)T, top, (int)E,
+                     stream));
   return p;
 }
 
@@ -764,24 +769,52 @@ Tensor Kernels::moe_up(const Tensor& h, const Tensor& w_up, const MoePlan& plan)
     throw EngineError("experts (up): input " + h.describe() + ", weights " + w_up.describe());
   const int64_t T = h.dim(0), N = w_up.dim(1);
   Tensor act = empty({plan.row_pair.dim(0), N});
-  call(fn_->moe_up(act.data, N, h.data, h.dim(1), w_up.data, plan.row_pair.data, plan.tile_expert.data, (int)T, plan.top, plan.experts, (int)N,
-                   (int)h.dim(1), stream));
+  call(fn_->moe_up(act.data, N, h.data, h.dim(1), w_up.data, plan.row_pair.data, plan.row_token.data, plan.tile_expert.data, (int)T, plan.top,
+                   plan.experts, (int)N, (int)h.dim(1), stream));
   return act;
 }
 
-Tensor Kernels::moe_down_sum(const Tensor& act, const Tensor& w_down, const MoePlan& plan, int64_t T) {
+Tensor Kernels::moe_down(const Tensor& act, const Tensor& w_down, const MoePlan& plan) {
   expect(act, "experts' activations", dtype_);
   expect(w_down, "experts' down weights", dtype_);
   if (act.shape.size() != 2 || w_down.shape.size() != 3 || w_down.dim(0) != plan.experts || w_down.dim(2) != act.dim(1) ||
-      act.dim(0) != plan.row_pair.dim(0) || plan.idx.dim(0) != T)
+      act.dim(0) != plan.row_pair.dim(0))
     throw EngineError("experts (down): activations " + act.describe() + ", weights " + w_down.describe());
-  const int64_t W = w_down.dim(1);
-  Tensor y = empty({act.dim(0), W}, DType::F32);
+  const int64_t W = w_down.dim(1), T = plan.idx.dim(0);
+  Tensor y = empty({act.dim(0), W});
   call(fn_->moe_down(y.data, act.data, act.dim(1), w_down.data, plan.row_pair.data, plan.tile_expert.data, (int)T, plan.top, plan.experts, (int)W,
                      (int)act.dim(1), stream));
+  return y;
+}
+
+Tensor Kernels::moe_sum(const Tensor& y, const MoePlan& plan) {
+  expect(y, "experts' outputs", dtype_);
+  if (y.shape.size() != 2 || y.dim(0) != plan.row_pair.dim(0)) throw EngineError("experts (sum): outputs " + y.describe());
+  const int64_t T = plan.idx.dim(0), W = y.dim(1);
   Tensor out = empty({T, W}, DType::F32);
   call(fn_->moe_combine(out.data, y.data, plan.wts.data, plan.pair_row.data, (int)T, (int)W, plan.top, stream));
   return out;
+}
+
+std::vector<int32_t> Kernels::moe_expert_rows(const MoePlan& plan) {
+  std::vector<int32_t> rows((size_t)plan.experts + 1);
+  hip_check(hipMemcpyAsync(rows.data(), plan.expert_start.data, rows.size() * sizeof(int32_t), hipMemcpyDeviceToHost, stream), "reading the experts' rows");
+  hip_check(hipStreamSynchronize(stream), "reading the experts' rows");
+  return rows;
+}
+
+void Kernels::relu_square(Tensor& x) {
+  expect(x, "activations", dtype_);
+  call(fn_->moe_relu_square(x.data, x.numel(), stream));
+}
+
+void Kernels::gemm_into(Tensor& out, const Tensor& act, const Tensor& w) {
+  expect(act, "activation", dtype_);
+  expect(w, "weight", dtype_);
+  expect(out, "product", dtype_);
+  if (act.shape.size() != 2 || w.shape.size() != 2 || out.shape.size() != 2 || act.dim(1) != w.dim(1) || out.dim(0) != act.dim(0) || out.dim(1) != w.dim(0))
+    throw EngineError("gemm: activation " + act.describe() + ", weight " + w.describe() + ", product " + out.describe());
+  call(fn_->gemm(out.data, act.data, w.data, (int)act.dim(0), (int)w.dim(0), (int)w.dim(1), act.dim(1), w.dim(0), 0, stream));
 }
 
 int Kernels::sample_scratch_words(int rows) const { return fn_->sample_scratch_words(rows); }

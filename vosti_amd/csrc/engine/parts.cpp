@@ -1045,10 +1045,39 @@ class RoutedExperts : public FeedForward {
     w_up_ = stack_rows(up).view({(int64_t)experts_, padded, hidden_});
     w_down_ = stack_rows(down).view({(int64_t)experts_, hidden_, padded});
   }
-  Tensor forward(const Tensor& x, StepContext&) override {
-    const Kernels::MoePlan plan = kernels.moe_route(x, router_, top_, weight_eps_);
-    return kernels.moe_down_sum(kernels.moe_up(x, w_up_, plan), w_down_, plan, x.dim(0));
+  Tensor forward(const Tensor& x, StepContext& ctx) override {
+    Kernels& k = kernels;
+    const Kernels::MoePlan plan = k.moe_route(x, router_, top_, weight_eps_);
+    const int64_t pairs = x.dim(0) * top_;
+    // Few rows an expert: grouped products over tiles of 16 rows, launched from numbers on the GPU alone (a recorded
+    // step always goes this way).  Many: the rows lie sorted by expert, so every expert's rows go through the engine's
+    // own matrix product, once the host knows how many each has.  The two ways give the same bits.
+    if (ctx.host->frozen || pairs < (int64_t)kRowsAnExpertForOwnProducts * experts_) return k.moe_sum(k.moe_down(k.moe_up(x, w_up_, plan), w_down_, plan), plan);
+    const std::vector<int32_t> start = k.moe_expert_rows(plan);
+    const int64_t rows = start.back(), ff = w_up_.dim(1);
+    const Tensor sorted = k.gather_rows(x, plan.row_token.rows(0, rows));
+    Tensor act = k.empty({plan.row_pair.dim(0), ff}), y = k.empty({plan.row_pair.dim(0), hidden_});
+    for (int pass = 0; pass < 2; ++pass) {
+      for (int e = 0; e < experts_; ++e) {
+        const int64_t first = start[e], n = start[e + 1] - first;
+        if (n <= 0) continue;
+        if (pass == 0) {
+          Tensor out = act.rows(first, n);
+          k.gemm_into(out, sorted.rows(first, n), w_up_.rows(e, 1).view({ff, hidden_}));
+        } else {
+          Tensor out = y.rows(first, n);
+          k.gemm_into(out, act.rows(first, n), w_down_.rows(e, 1).view({hidden_, ff}));
+        }
+      }
+      if (pass == 0) {
+        Tensor used = act.rows(0, rows);
+        k.relu_square(used);
+      }
+    }
+    return k.moe_sum(y, plan);
   }
+  // The second way reads a count from the GPU in the middle of a step; a recorded step never takes it.
+  static constexpr int kRowsAnExpertForOwnProducts = 64;
 
  private:
   int64_t hidden_, inter_;

@@ -5,9 +5,9 @@
 // where x [P] is the head's input, B and C [N] the token's input and output vectors.  Everything here is 32-bit; the
 // projection that feeds dt arrives as elements, x, B and C as the 32-bit output of the short convolution.
 //
-// A sequence's tokens are walked in order by one workgroup per (sequence, head, block of 32 value columns).  A column's
-// state is spread over 8 neighbouring lanes, each holding DR consecutive state rows in registers; a token's read-out is
-// the sum over a lane's rows in ascending order and then a butterfly over the 8 lanes, whatever the step's cut: the
+// A sequence's tokens are walked in order by one workgroup per (sequence, head, block of value columns).  A column's
+// state is spread over R neighbouring lanes, each holding DR consecutive state rows in registers; a token's read-out is
+// the sum over a lane's rows in ascending order and then a butterfly over the R lanes, whatever the step's cut: the
 // state that a step leaves in memory (per head [P][N], 32-bit) is what the next step starts from, bit for bit.  The
 // inputs of a chunk of tokens go through LDS: the next chunk's are read from global memory into registers before this
 // chunk is walked and written to the other LDS buffer after it (one barrier a chunk).
@@ -17,8 +17,6 @@
 #include "vec.h"
 
 #define SSM_THREADS 256
-#define SSM_LANES 8
-#define SSM_COLS (SSM_THREADS / SSM_LANES)
 #define SSM_CHUNK 16
 
 struct SsmArgs {
@@ -42,20 +40,22 @@ struct SsmArgs {
 
 __device__ __forceinline__ float ssm_softplus(float z) { return z > 20.f ? z : log1pf(expf(z)); }
 
-template <int DR, int ROUNDS>
+// R lanes share a value column, each with DR consecutive state rows; a workgroup has 256 / R columns.  In LDS the
+// state rows are padded with zeros to R * DR, so that no lane has to ask whether a row exists.
+template <int R, int DR, int ROUNDS>
 __global__ __launch_bounds__(SSM_THREADS) void ssm_scan_kernel(SsmArgs a) {
   extern __shared__ float lds[];
+  constexpr int COLS = SSM_THREADS / R, NP = R * DR;
+  // A token's row in LDS: B [NP], C [NP], the workgroup's x columns [COLS], dt, the decay, and two to a whole vector.
+  constexpr int L1 = 2 * NP + COLS + 1, RS = 2 * NP + COLS + 4;
   const int s = blockIdx.x, h = blockIdx.y, tid = threadIdx.x;
   const int N = a.N, P = a.P, g = h / (a.H / a.G);
-  const int col = tid / SSM_LANES, r = tid % SSM_LANES;
-  const int p = blockIdx.z * SSM_COLS + col;
+  const int col = tid / R, r = tid % R;
+  const int p = blockIdx.z * COLS + col;
   const bool col_ok = p < P;
   const int first = a.cu_q[s], n_tok = a.cu_q[s + 1] - first;
   if (n_tok <= 0) return;
   const bool fresh = a.positions[first] == 0;
-  // A token's row in LDS: B [N], C [N], the workgroup's x columns [SSM_COLS], dt, the decay.
-  const int L1 = 2 * N + SSM_COLS + 1, RS = L1 + 1;
-  float* buf[2] = {lds, lds + SSM_CHUNK * RS};
 
   float S[DR];
   float* st = a.state + (int64_t)a.slots[s] * a.state_stride + ((int64_t)h * P + (col_ok ? p : 0)) * N;
@@ -73,20 +73,21 @@ __global__ __launch_bounds__(SSM_THREADS) void ssm_scan_kernel(SsmArgs a) {
 #pragma unroll
     for (int rd = 0; rd < ROUNDS; ++rd) {
       const int e = tid + rd * SSM_THREADS;
+      // Where this thread's element of a token's row comes from: -1 nowhere (padding), else an offset from the row's start.
+      int64_t src = -1;
+      bool is_dt = false;
+      if (e < NP) { if (e < N) src = a.b_col + g * N + e; }
+      else if (e < 2 * NP) { if (e - NP < N) src = a.c_col + g * N + (e - NP); }
+      else if (e < 2 * NP + COLS) { if ((int)(blockIdx.z * COLS) + (e - 2 * NP) < P) src = h * P + blockIdx.z * COLS + (e - 2 * NP); }
+      else if (e == L1 - 1) is_dt = true;
 #pragma unroll
       for (int i = 0; i < SSM_CHUNK; ++i) {
         const int t = c * SSM_CHUNK + i;
         float v = 0.f;
-        if (t < n_tok && e < L1) {
+        if (t < n_tok) {
           const int64_t row = (int64_t)(first + t);
-          if (e < N) v = a.xbc[row * a.ldx + a.b_col + g * N + e];
-          else if (e < 2 * N) v = a.xbc[row * a.ldx + a.c_col + g * N + (e - N)];
-          else if (e < 2 * N + SSM_COLS) {
-            const int pc = blockIdx.z * SSM_COLS + (e - 2 * N);
-            if (pc < P) v = a.xbc[row * a.ldx + h * P + pc];
-          } else {
-            v = to_f32(a.dt[row * a.lddt + h]);
-          }
+          if (src >= 0) v = a.xbc[row * a.ldx + src];
+          else if (is_dt) v = to_f32(a.dt[row * a.lddt + h]);
         }
         reg[rd][i] = v;
       }
@@ -112,32 +113,42 @@ __global__ __launch_bounds__(SSM_THREADS) void ssm_scan_kernel(SsmArgs a) {
 
   const int chunks = (n_tok + SSM_CHUNK - 1) / SSM_CHUNK;
   fetch(0);
-  stage(buf[0]);
+  stage(lds);
   __syncthreads();
   for (int c = 0; c < chunks; ++c) {
     if (c + 1 < chunks) fetch(c + 1);
-    const float* cur = buf[c & 1];
+    const float* cur = lds + (c & 1) * (SSM_CHUNK * RS);
     const int m = min(SSM_CHUNK, n_tok - c * SSM_CHUNK);
+    float* yout = a.y + (int64_t)(first + c * SSM_CHUNK) * ((int64_t)a.H * P) + (int64_t)h * P + p;
     for (int i = 0; i < m; ++i) {
       const float* row = cur + i * RS;
-      const float xv = row[2 * N + col], dtv = row[L1 - 1], dA = row[L1];
+      const float xv = row[2 * NP + col], dtv = row[L1 - 1], dA = row[L1];
       const float dx = dtv * xv;
+      const float* Bp = row + r * DR;
+      const float* Cp = row + NP + r * DR;
       float acc = 0.f;
+      if constexpr (DR % 4 == 0) {
 #pragma unroll
-      for (int j = 0; j < DR; ++j) {
-        const int n = r * DR + j;
-        const bool in = n < N;
-        const int nn = in ? n : 0;
-        const float Bn = in ? row[nn] : 0.f, Cn = in ? row[N + nn] : 0.f;
-        S[j] = __builtin_fmaf(dA, S[j], dx * Bn);
-        acc = __builtin_fmaf(S[j], Cn, acc);
+        for (int q = 0; q < DR / 4; ++q) {
+          const f32x4 b4 = *reinterpret_cast<const f32x4*>(Bp + 4 * q), c4 = *reinterpret_cast<const f32x4*>(Cp + 4 * q);
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            S[4 * q + j] = __builtin_fmaf(dA, S[4 * q + j], dx * b4[j]);
+            acc = __builtin_fmaf(S[4 * q + j], c4[j], acc);
+          }
+        }
+      } else {
+#pragma unroll
+        for (int j = 0; j < DR; ++j) {
+          S[j] = __builtin_fmaf(dA, S[j], dx * Bp[j]);
+          acc = __builtin_fmaf(S[j], Cp[j], acc);
+        }
       }
-      acc = acc + __shfl_xor(acc, 1, VK_WAVE);
-      acc = acc + __shfl_xor(acc, 2, VK_WAVE);
-      acc = acc + __shfl_xor(acc, 4, VK_WAVE);
-      if (r == 0 && col_ok) a.y[(int64_t)(first + c * SSM_CHUNK + i) * ((int64_t)a.H * P) + (int64_t)h * P + p] = acc + Dh * xv;
+#pragma unroll
+      for (int off = 1; off < R; off <<= 1) acc = acc + __shfl_xor(acc, off, VK_WAVE);
+      if (r == 0 && col_ok) yout[(int64_t)i * ((int64_t)a.H * P)] = acc + Dh * xv;
     }
-    if (c + 1 < chunks) stage(buf[(c + 1) & 1]);
+    if (c + 1 < chunks) stage(lds + ((c + 1) & 1) * (SSM_CHUNK * RS));
     __syncthreads();
   }
   if (col_ok) {
@@ -193,33 +204,33 @@ int vk_ssm_scan(float* y, const float* xbc, int64_t ldx, int b_col, int c_col, c
   VK_REQUIRE(b_col >= H * P && c_col >= 0 && ldx >= (int64_t)std::max(b_col, c_col) + (int64_t)G * N && lddt >= H,
              "state-space scan: the rows do not hold the inputs");
   VK_REQUIRE(state_stride >= (int64_t)H * P * N, "state-space scan: the state does not hold the heads");
-  VK_REQUIRE(H <= 65535 && (P + SSM_COLS - 1) / SSM_COLS <= 65535, "state-space scan: too many heads or columns");
+  VK_REQUIRE(H <= 65535, "state-space scan: too many heads");
   if (S == 0) return 0;
   SsmArgs a;
   a.y = y; a.xbc = xbc; a.ldx = ldx; a.b_col = b_col; a.c_col = c_col; a.dt = dt; a.lddt = lddt; a.dt_bias = dt_bias; a.A_log = A_log; a.D = D;
   a.w_is_f32 = w_is_f32; a.state = state; a.state_stride = state_stride; a.cu_q = cu_q; a.positions = positions; a.slots = slots;
   a.H = H; a.G = G; a.N = N; a.P = P;
-  const dim3 grid(S, H, (P + SSM_COLS - 1) / SSM_COLS);
-  const int L1 = 2 * N + SSM_COLS + 1;
-  const size_t smem = (size_t)2 * SSM_CHUNK * (L1 + 1) * sizeof(float);
-  const int rounds = (L1 + SSM_THREADS - 1) / SSM_THREADS;
-  const int dr = (N + SSM_LANES - 1) / SSM_LANES;
-  // More than 64 KB of LDS has to be asked for once per kernel.
-#define SSM_SCAN(DR, ROUNDS)                                                                                                  \
-  do {                                                                                                                        \
-    static bool raised = false;                                                                                               \
-    if (!raised && smem > 48 * 1024) {                                                                                        \
-      (void)hipFuncSetAttribute((const void*)ssm_scan_kernel<DR, ROUNDS>, hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024); \
-      raised = true;                                                                                                          \
-    }                                                                                                                         \
-    ssm_scan_kernel<DR, ROUNDS><<<grid, SSM_THREADS, smem, st>>>(a);                                                          \
+  // Lanes a column and rows a lane: 16 lanes from 128 state rows on (more workgroups, shorter sums a token), else 8.
+#define SSM_SCAN(R, DR, ROUNDS)                                                                                                  \
+  do {                                                                                                                           \
+    constexpr int cols = SSM_THREADS / (R);                                                                                      \
+    const size_t smem = (size_t)2 * SSM_CHUNK * (2 * (R) * (DR) + cols + 4) * sizeof(float);                                      \
+    static_assert((2 * (R) * (DR) + cols + 1 + SSM_THREADS - 1) / SSM_THREADS <= (ROUNDS), "a round more is needed");            \
+    static bool raised = false;                                                                                                  \
+    if (!raised && smem > 48 * 1024) {                                                                                           \
+      (void)hipFuncSetAttribute((const void*)ssm_scan_kernel<R, DR, ROUNDS>, hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024); \
+      raised = true;                                                                                                             \
+    }                                                                                                                            \
+    VK_REQUIRE((P + cols - 1) / cols <= 65535, "state-space scan: too many columns");                                            \
+    ssm_scan_kernel<R, DR, ROUNDS><<<dim3(S, H, (P + cols - 1) / cols), SSM_THREADS, smem, st>>>(a);                             \
   } while (0)
-  if (dr <= 1) SSM_SCAN(1, 1);
-  else if (dr <= 2) SSM_SCAN(2, 1);
-  else if (dr <= 4) SSM_SCAN(4, 1);
-  else if (dr <= 8) SSM_SCAN(8, 1);
-  else if (dr <= 16) { if (rounds <= 1) SSM_SCAN(16, 1); else SSM_SCAN(16, 2); }
-  else { if (rounds <= 2) SSM_SCAN(32, 2); else SSM_SCAN(32, 3); }
+  if (N <= 8) SSM_SCAN(8, 1, 1);
+  else if (N <= 16) SSM_SCAN(8, 2, 1);
+  else if (N <= 32) SSM_SCAN(8, 4, 1);
+  else if (N <= 64) SSM_SCAN(8, 8, 1);
+  else if (N < 128) SSM_SCAN(8, 16, 2);
+  else if (N == 128) SSM_SCAN(16, 8, 2);
+  else SSM_SCAN(16, 16, 3);
 #undef SSM_SCAN
   return vk_check_launch("state-space scan");
 }

@@ -243,6 +243,47 @@ __global__ __launch_bounds__(STREAM_THREADS) void stream_pair_norm_kernel(float*
   }
 }
 
+// The same for rows of whole 16-byte vectors that fit a workgroup's registers (thread t owns the vectors t, t + 256, ...).
+template <int NV>
+__global__ __launch_bounds__(STREAM_THREADS) void stream_pair_norm_vec_kernel(float* __restrict__ out, const elem_t* __restrict__ a,
+                                                                              const void* __restrict__ wa, const elem_t* __restrict__ b,
+                                                                              const void* __restrict__ wb, int w_is_f32, int H, float eps,
+                                                                              float ca, float cb) {
+  __shared__ float red_a[4], red_b[4];
+  const int64_t base = (int64_t)blockIdx.x * H;
+  const int nvec = H / 4;
+  f32x4 va[NV], vb[NV];
+  float pa = 0.f, pb = 0.f;
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const int c = threadIdx.x + j * STREAM_THREADS;
+    va[j] = vb[j] = f32x4{0.f, 0.f, 0.f, 0.f};
+    if (c < nvec) {
+      const elem_t *p = a + base + 4 * c, *q = b + base + 4 * c;
+      va[j] = f32x4{to_f32(p[0]), to_f32(p[1]), to_f32(p[2]), to_f32(p[3])};
+      vb[j] = f32x4{to_f32(q[0]), to_f32(q[1]), to_f32(q[2]), to_f32(q[3])};
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      pa = pa + va[j][e] * va[j][e];
+      pb = pb + vb[j][e] * vb[j][e];
+    }
+  }
+  const float ra = rsqrtf(stream_block_sum(pa, red_a) / (float)H + eps);
+  const float rb = rsqrtf(stream_block_sum(pb, red_b) / (float)H + eps);
+#pragma unroll
+  for (int j = 0; j < NV; ++j) {
+    const int c = threadIdx.x + j * STREAM_THREADS;
+    if (c < nvec) {
+      f32x4 o;
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        o[e] = ca * ((va[j][e] * ra) * load_weight(wa, w_is_f32, 4 * c + e)) + cb * ((vb[j][e] * rb) * load_weight(wb, w_is_f32, 4 * c + e));
+      *reinterpret_cast<f32x4*>(out + base + 4 * c) = o;
+    }
+  }
+}
+
 extern "C" {
 
 int vk_embed_sinusoid(float* out, const elem_t* table, const int32_t* ids, const int32_t* positions, const float* inv_freq, int T,
@@ -331,7 +372,14 @@ int vk_stream_pair_norm(float* out, const elem_t* a, const void* wa, const elem_
                         float ca, float cb, hipStream_t st) {
   VK_REQUIRE(rows >= 0 && H > 0 && eps >= 0.f, "pair norm: bad sizes rows=%d H=%d", rows, H);
   if (rows == 0) return 0;
-  stream_pair_norm_kernel<<<rows, STREAM_THREADS, 0, st>>>(out, a, wa, b, wb, w_is_f32, H, eps, ca, cb);
+  const int nv = (H / 4 + STREAM_THREADS - 1) / STREAM_THREADS;
+  if (H % 4 == 0 && nv <= 8 && (uintptr_t)out % 16 == 0) {
+#define PAIR_VEC(NV) stream_pair_norm_vec_kernel<NV><<<rows, STREAM_THREADS, 0, st>>>(out, a, wa, b, wb, w_is_f32, H, eps, ca, cb)
+    if (nv <= 1) PAIR_VEC(1); else if (nv <= 2) PAIR_VEC(2); else if (nv <= 4) PAIR_VEC(4); else PAIR_VEC(8);
+#undef PAIR_VEC
+  } else {
+    stream_pair_norm_kernel<<<rows, STREAM_THREADS, 0, st>>>(out, a, wa, b, wb, w_is_f32, H, eps, ca, cb);
+  }
   return vk_check_launch("pair norm");
 }
 
