@@ -69,6 +69,31 @@ __device__ __forceinline__ float lane_xor32(float v) {
   return __builtin_bit_cast(float, (threadIdx.x & 32) ? r[0] : r[1]);
 }
 
+// The sum over the R neighbouring lanes of an aligned group, in every lane of the group: a butterfly whose steps stay
+// in the vector unit (quad permutes, the mirrors of a half row and of a row, the swaps of rows and halves).  The order
+// of the additions is fixed by R.
+__device__ __forceinline__ float dpp_f(float v, int ctrl_tag) {
+  const int x = __builtin_bit_cast(int, v);
+  int y;
+  switch (ctrl_tag) {
+    case 0: y = __builtin_amdgcn_update_dpp(x, x, 0xB1, 0xF, 0xF, false); break;    // quad_perm [1, 0, 3, 2]
+    case 1: y = __builtin_amdgcn_update_dpp(x, x, 0x4E, 0xF, 0xF, false); break;    // quad_perm [2, 3, 0, 1]
+    case 2: y = __builtin_amdgcn_update_dpp(x, x, 0x141, 0xF, 0xF, false); break;   // row_half_mirror
+    default: y = __builtin_amdgcn_update_dpp(x, x, 0x140, 0xF, 0xF, false); break;  // row_mirror
+  }
+  return __builtin_bit_cast(float, y);
+}
+template <int R>
+__device__ __forceinline__ float group_sum(float v) {
+  if (R >= 2) v = v + dpp_f(v, 0);
+  if (R >= 4) v = v + dpp_f(v, 1);
+  if (R >= 8) v = v + dpp_f(v, 2);
+  if (R >= 16) v = v + dpp_f(v, 3);
+  if (R >= 32) v = v + lane_xor16(v);
+  if (R >= 64) v = v + lane_xor32(v);
+  return v;
+}
+
 __device__ __forceinline__ float wave_max_xor(float v) {
 #pragma unroll
   for (int off = 32; off >= 1; off >>= 1) v = fmaxf(v, __shfl_xor(v, off, VK_WAVE));

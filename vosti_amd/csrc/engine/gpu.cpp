@@ -122,9 +122,10 @@ struct Kernels::Fn {
   int (*stream_pair_norm)(P, CP, CP, CP, CP, int, int, int, float, float, float, hipStream_t);
   int (*ssm_scan)(P, CP, int64_t, int, int, CP, int64_t, CP, CP, CP, int, P, int64_t, CP, CP, CP, int, int, int, int, int, hipStream_t);
   int (*ssm_gate_norm)(P, int64_t, CP, CP, int64_t, CP, int, int, int, int, float, hipStream_t);
-  int (*moe_max_tiles)(int, int, int);
+  int (*moe_max_tiles)(int, int, int, int);
+  int (*gemm_grouped)(P, CP, CP, int, int, int, int64_t, int64_t, CP, int64_t, hipStream_t);
   int (*moe_route)(P, P, P, CP, CP, int, int, int, int, float, hipStream_t);
-  int (*moe_plan)(CP, P, P, P, P, P, int, int, int, hipStream_t);
+  int (*moe_plan)(CP, P, P, P, P, P, int, int, int, int, hipStream_t);
   int (*moe_up)(P, int64_t, CP, int64_t, CP, CP, CP, CP, int, int, int, int, int, hipStream_t);
   int (*moe_down)(P, CP, int64_t, CP, CP, CP, int, int, int, int, int, hipStream_t);
   int (*moe_combine)(P, CP, CP, CP, int, int, int, hipStream_t);
@@ -165,7 +166,7 @@ Kernels::Kernels(const std::string& lib_dir, const std::string& name) : name_(na
   VK(qkv_post_angles, "vk_qkv_post_angles"); VK(embed_scaled, "vk_embed_scaled"); VK(stream_add, "vk_stream_add");
   VK(stream_pair_norm, "vk_stream_pair_norm"); VK(ssm_scan, "vk_ssm_scan"); VK(ssm_gate_norm, "vk_ssm_gate_norm");
   VK(moe_max_tiles, "vk_moe_max_tiles"); VK(moe_route, "vk_moe_route"); VK(moe_plan, "vk_moe_plan"); VK(moe_up, "vk_moe_up");
-  VK(moe_down, "vk_moe_down"); VK(moe_combine, "vk_moe_combine"); VK(moe_relu_square, "vk_moe_relu_square");
+  VK(moe_down, "vk_moe_down"); VK(moe_combine, "vk_moe_combine"); VK(moe_relu_square, "vk_moe_relu_square"); VK(gemm_grouped, "vk_gemm_grouped");
 #undef VK
   segment_keys_ = fn_->attn_segment_keys();
   item_rows_ = fn_->attn_item_rows();
@@ -738,34 +739,37 @@ Tensor Kernels::ssm_gate_norm(const Tensor& y, const Tensor& proj, int64_t z_col
 }
 
 // ------------------------------------------------------------------------------ mixture of experts
-Kernels::MoePlan Kernels::moe_route(const Tensor& h, const Tensor& router, int top, float weight_eps) {
+Kernels::MoePlan Kernels::moe_route(const Tensor& h, const Tensor& router, int top, float weight_eps, int tile_rows) {
   expect(h, "router input", dtype_);
   expect(router, "router weight", dtype_);
   if (h.shape.size() != 2 || router.shape.size() != 2 || router.dim(1) != h.dim(1) || top < 1 || top > router.dim(0))
     throw EngineError("router: input " + h.describe() + ", weight " + router.describe() + ", top " + std::to_string(top));
   const int64_t T = h.dim(0), E = router.dim(0);
   MoePlan p;
+  if (tile_rows != 16 && tile_rows != 128) throw EngineError("router: tiles of " + std::to_string(tile_rows) + " rows");
   p.top = top;
   p.experts = (int)E;
-  const int64_t tiles = fn_->moe_max_tiles((int)T, top, (int)E);
+  p.tile_rows = tile_rows;
+  const int64_t tiles = fn_->moe_max_tiles((int)T, top, (int)E, tile_rows);
   p.idx = empty({T, top}, DType::I32);
   p.wts = empty({T, top}, DType::F32);
-  p.row_pair = empty({tiles * 16}, DType::I32);
-  p.row_token = empty({tiles * 16}, DType::I32);
+  p.row_pair = empty({tiles * tile_rows}, DType::I32);
+  p.row_token = empty({tiles * tile_rows}, DType::I32);
   p.pair_row = empty({T * top}, DType::I32);
   p.tile_expert = empty({tiles}, DType::I32);
   p.expert_start = empty({E + 1}, DType::I32);
   Tensor logits = empty({T, E}, DType::F32);
   call(fn_->moe_route(p.idx.data, p.wts.data, logits.data, h.data, router.data, (int)T, (int)h.dim(1), (int)E, top, weight_eps, stream));
   call(fn_->moe_plan(p.idx.data, p.row_pair.data, p.row_token.data, p.pair_row.data, p.tile_expert.data, p.expert_start.data, (int)T, top, (int)E,
-                     stream));
+                     tile_rows, stream));
   return p;
 }
 
 Tensor Kernels::moe_up(const Tensor& h, const Tensor& w_up, const MoePlan& plan) {
   expect(h, "experts' input", dtype_);
   expect(w_up, "experts' up weights", dtype_);
-  if (h.shape.size() != 2 || w_up.shape.size() != 3 || w_up.dim(0) != plan.experts || w_up.dim(2) != h.dim(1) || plan.idx.dim(0) != h.dim(0))
+  if (h.shape.size() != 2 || w_up.shape.size() != 3 || w_up.dim(0) != plan.experts || w_up.dim(2) != h.dim(1) || plan.idx.dim(0) != h.dim(0) ||
+      plan.tile_rows != 16)
     throw EngineError("experts (up): input " + h.describe() + ", weights " + w_up.describe());
   const int64_t T = h.dim(0), N = w_up.dim(1);
   Tensor act = empty({plan.row_pair.dim(0), N});
@@ -778,7 +782,7 @@ Tensor Kernels::moe_down(const Tensor& act, const Tensor& w_down, const MoePlan&
   expect(act, "experts' activations", dtype_);
   expect(w_down, "experts' down weights", dtype_);
   if (act.shape.size() != 2 || w_down.shape.size() != 3 || w_down.dim(0) != plan.experts || w_down.dim(2) != act.dim(1) ||
-      act.dim(0) != plan.row_pair.dim(0))
+      act.dim(0) != plan.row_pair.dim(0) || plan.tile_rows != 16)
     throw EngineError("experts (down): activations " + act.describe() + ", weights " + w_down.describe());
   const int64_t W = w_down.dim(1), T = plan.idx.dim(0);
   Tensor y = empty({act.dim(0), W});
@@ -796,25 +800,23 @@ Tensor Kernels::moe_sum(const Tensor& y, const MoePlan& plan) {
   return out;
 }
 
-std::vector<int32_t> Kernels::moe_expert_rows(const MoePlan& plan) {
-  std::vector<int32_t> rows((size_t)plan.experts + 1);
-  hip_check(hipMemcpyAsync(rows.data(), plan.expert_start.data, rows.size() * sizeof(int32_t), hipMemcpyDeviceToHost, stream), "reading the experts' rows");
-  hip_check(hipStreamSynchronize(stream), "reading the experts' rows");
-  return rows;
-}
-
 void Kernels::relu_square(Tensor& x) {
   expect(x, "activations", dtype_);
   call(fn_->moe_relu_square(x.data, x.numel(), stream));
 }
 
-void Kernels::gemm_into(Tensor& out, const Tensor& act, const Tensor& w) {
+bool Kernels::gemm_grouped_takes(int64_t K) const { return K % (dtype_ == DType::BF16 ? 64 : 32) == 0; }
+
+Tensor Kernels::gemm_grouped(const Tensor& act, const Tensor& w, const Tensor& block_weights) {
   expect(act, "activation", dtype_);
-  expect(w, "weight", dtype_);
-  expect(out, "product", dtype_);
-  if (act.shape.size() != 2 || w.shape.size() != 2 || out.shape.size() != 2 || act.dim(1) != w.dim(1) || out.dim(0) != act.dim(0) || out.dim(1) != w.dim(0))
-    throw EngineError("gemm: activation " + act.describe() + ", weight " + w.describe() + ", product " + out.describe());
-  call(fn_->gemm(out.data, act.data, w.data, (int)act.dim(0), (int)w.dim(0), (int)w.dim(1), act.dim(1), w.dim(0), 0, stream));
+  expect(w, "weights", dtype_);
+  if (act.shape.size() != 2 || w.shape.size() != 3 || act.dim(1) != w.dim(2) || act.dim(0) % 128 || !gemm_grouped_takes(act.dim(1)))
+    throw EngineError("grouped gemm: activation " + act.describe() + ", weights " + w.describe());
+  expect(block_weights, "the blocks' matrices", DType::I32, {act.dim(0) / 128});
+  Tensor out = empty({act.dim(0), w.dim(1)});
+  call(fn_->gemm_grouped(out.data, act.data, w.data, (int)act.dim(0), (int)w.dim(1), (int)w.dim(2), act.dim(1), w.dim(1), block_weights.data,
+                         w.dim(1) * w.dim(2), stream));
+  return out;
 }
 
 int Kernels::sample_scratch_words(int rows) const { return fn_->sample_scratch_words(rows); }

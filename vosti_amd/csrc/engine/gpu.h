@@ -192,20 +192,21 @@ class Kernels {
     Tensor idx, wts;                            // [T, top]
     Tensor row_pair, row_token, pair_row, tile_expert;
     Tensor expert_start;                        // [experts + 1] on the GPU: every expert's first row, and the rows in use
-    int top = 0, experts = 0;
+    int top = 0, experts = 0, tile_rows = 16;   // an expert's rows are padded to whole tiles of this many
   };
-  MoePlan moe_route(const Tensor& h, const Tensor& router, int top, float weight_eps);
+  // tile_rows 16: for moe_up / moe_down; 128: for gemm_grouped, whose blocks are the plan's tiles.
+  MoePlan moe_route(const Tensor& h, const Tensor& router, int top, float weight_eps, int tile_rows = 16);
   // relu(h W_up^T)^2 of every (token, choice) in the plan's rows; w_up [E, ff, width]; result [rows, ff] elements.
   Tensor moe_up(const Tensor& h, const Tensor& w_up, const MoePlan& plan);
   // The chosen experts' down projections of the plan's rows, [rows, width] elements; w_down [E, width, ff].
   Tensor moe_down(const Tensor& act, const Tensor& w_down, const MoePlan& plan);
   // The weighted sum of a token's rows, floats [T, width].
   Tensor moe_sum(const Tensor& y, const MoePlan& plan);
-  // expert_start on the host; waits for the stream.
-  std::vector<int32_t> moe_expert_rows(const MoePlan& plan);
+  // act [M, K] in blocks of 128 rows, block b times the matrix block_weights[b] of w [matrices, N, K] (negative: the
+  // block is skipped); [M, N] elements, the bits gemm gives for the same rows and matrix.  K in whole pairs of slabs.
+  Tensor gemm_grouped(const Tensor& act, const Tensor& w, const Tensor& block_weights);
+  bool gemm_grouped_takes(int64_t K) const;
   void relu_square(Tensor& x);                 // x <- max(x, 0)^2
-  // out = act @ w^T into rows the caller owns (out [M, N], act [M, K], w [N, K], all whole rows of their tensors).
-  void gemm_into(Tensor& out, const Tensor& act, const Tensor& w);
   int segment_keys() const { return segment_keys_; }
   int item_rows() const { return item_rows_; }
 

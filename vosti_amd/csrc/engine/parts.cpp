@@ -1015,8 +1015,8 @@ class PairMean : public Mixer {
 // A mixture of `experts` small feed-forward layers without biases, W_down max(W_up h, 0)^2, of which every token uses
 // `top`: router logits W_router h in 32-bit, a softmax over all experts, the `top` largest scores, divided by their
 // sum plus weight_eps; the output is the weighted sum of the chosen experts' outputs, in 32-bit.  The experts' weights
-// lie stacked, [experts, ff, width] and [experts, width, ff] (ff padded to whole 16-byte vectors with zeros), and the
-// two projections run as grouped products over the (token, choice) pairs sorted by expert (moe.hip).
+// lie stacked, [experts, ff, width] and [experts, width, ff] (ff padded to a multiple of 64 with zeros), and the two
+// projections run as grouped products over the (token, choice) pairs sorted by expert (moe.hip, gemm.hip).
 class RoutedExperts : public FeedForward {
  public:
   RoutedExperts(const PartSpec& s, Kernels& k)
@@ -1035,7 +1035,7 @@ class RoutedExperts : public FeedForward {
   }
   void load(std::map<std::string, Tensor>& t) override {
     router_ = need(t, "router.weight");
-    const int64_t padded = round_up(inter_, 8);
+    const int64_t padded = round_up(inter_, 64);              // whole pairs of slabs, so that the tile product takes it
     std::vector<Tensor> up, down;
     for (int e = 0; e < experts_; ++e) {
       up.push_back(pad_matrix(need(t, "experts." + std::to_string(e) + ".up_proj.weight"), padded, hidden_));
@@ -1045,39 +1045,22 @@ class RoutedExperts : public FeedForward {
     w_up_ = stack_rows(up).view({(int64_t)experts_, padded, hidden_});
     w_down_ = stack_rows(down).view({(int64_t)experts_, hidden_, padded});
   }
-  Tensor forward(const Tensor& x, StepContext& ctx) override {
+  Tensor forward(const Tensor& x, StepContext&) override {
     Kernels& k = kernels;
-    const Kernels::MoePlan plan = k.moe_route(x, router_, top_, weight_eps_);
     const int64_t pairs = x.dim(0) * top_;
-    // Few rows an expert: grouped products over tiles of 16 rows, launched from numbers on the GPU alone (a recorded
-    // step always goes this way).  Many: the rows lie sorted by expert, so every expert's rows go through the engine's
-    // own matrix product, once the host knows how many each has.  The two ways give the same bits.
-    if (ctx.host->frozen || pairs < (int64_t)kRowsAnExpertForOwnProducts * experts_) return k.moe_sum(k.moe_down(k.moe_up(x, w_up_, plan), w_down_, plan), plan);
-    const std::vector<int32_t> start = k.moe_expert_rows(plan);
-    const int64_t rows = start.back(), ff = w_up_.dim(1);
-    const Tensor sorted = k.gather_rows(x, plan.row_token.rows(0, rows));
-    Tensor act = k.empty({plan.row_pair.dim(0), ff}), y = k.empty({plan.row_pair.dim(0), hidden_});
-    for (int pass = 0; pass < 2; ++pass) {
-      for (int e = 0; e < experts_; ++e) {
-        const int64_t first = start[e], n = start[e + 1] - first;
-        if (n <= 0) continue;
-        if (pass == 0) {
-          Tensor out = act.rows(first, n);
-          k.gemm_into(out, sorted.rows(first, n), w_up_.rows(e, 1).view({ff, hidden_}));
-        } else {
-          Tensor out = y.rows(first, n);
-          k.gemm_into(out, act.rows(first, n), w_down_.rows(e, 1).view({hidden_, ff}));
-        }
-      }
-      if (pass == 0) {
-        Tensor used = act.rows(0, rows);
-        k.relu_square(used);
-      }
+    // Few rows an expert: products over tiles of 16 rows that stream an expert's weights once a tile.  Many (prompts):
+    // the rows are sorted by expert into blocks of 128 and go through the engine's tile product, every block with its
+    // expert's matrix.  Both are launched from numbers on the GPU alone and give the same bits.
+    if (pairs < (int64_t)kRowsAnExpertForTiles * experts_ || !k.gemm_grouped_takes(hidden_) || !k.gemm_grouped_takes(w_up_.dim(1))) {
+      const Kernels::MoePlan plan = k.moe_route(x, router_, top_, weight_eps_);
+      return k.moe_sum(k.moe_down(k.moe_up(x, w_up_, plan), w_down_, plan), plan);
     }
-    return k.moe_sum(y, plan);
+    const Kernels::MoePlan plan = k.moe_route(x, router_, top_, weight_eps_, 128);
+    Tensor act = k.gemm_grouped(k.gather_rows(x, plan.row_token), w_up_, plan.tile_expert);
+    k.relu_square(act);
+    return k.moe_sum(k.gemm_grouped(act, w_down_, plan.tile_expert), plan);
   }
-  // The second way reads a count from the GPU in the middle of a step; a recorded step never takes it.
-  static constexpr int kRowsAnExpertForOwnProducts = 64;
+  static constexpr int kRowsAnExpertForTiles = 32;
 
  private:
   int64_t hidden_, inter_;

@@ -560,7 +560,8 @@ __device__ __forceinline__ void wait_vmcnt_n() {             // vmcnt(N_), N_ be
 template <int S, bool WHOLE, bool SWIGLU, int FNW = 4, int PFD = 0>
 __global__ __launch_bounds__(256, 2) void gemm_pipe_kernel(elem_t* __restrict__ out, const elem_t* __restrict__ act,
                                                         const elem_t* __restrict__ w, int M, int N, int K,
-                                                        int64_t lda, int64_t ldo, int out_vec_ok, int band_w) {
+                                                        int64_t lda, int64_t ldo, int out_vec_ok, int band_w,
+                                                        const int32_t* __restrict__ block_weights, int64_t weights_stride) {
   static_assert(FNW >= 2 && FNW <= 5 && (FNW == 4 || !SWIGLU), "two to five weight fragments per wave; four with SwiGLU");
   static_assert(PFD == 0 || FNW == 2 || FNW == 4, "the touch-ahead wants a wave's 64 rows to be of one kind");
   constexpr int BN = 32 * FNW;                          // weight rows of the workgroup
@@ -584,6 +585,13 @@ __global__ __launch_bounds__(256, 2) void gemm_pipe_kernel(elem_t* __restrict__ 
     const int w_here = min(band_w, (int)gridDim.x - band * band_w);
     mb = r / w_here;
     nb = band * band_w + (r - mb * w_here);
+  }
+  // A grouped product: every block of 128 rows has a weight matrix of its own, block_weights[mb] of several that lie
+  // weights_stride elements apart (a negative number: the block is not in use).
+  if (block_weights != nullptr) {
+    const int which = block_weights[mb];
+    if (which < 0) return;
+    w += (int64_t)which * weights_stride;
   }
   const int n_blk = nb * (SWIGLU ? 64 : BN), m_blk = mb * 128;
   const int ntiles = K / (2 * VK_SLAB);
@@ -775,7 +783,7 @@ static const int pipe_band_blocks = 64;
 
 template <int S, bool SWIGLU = false, int FNW = 4>
 static int launch_pipe(elem_t* out, const elem_t* act, const elem_t* w, int M, int N, int K, int64_t lda, int64_t ldo,
-                       int vec_ok, hipStream_t st) {
+                       int vec_ok, hipStream_t st, const int32_t* block_weights = nullptr, int64_t weights_stride = 0) {
   constexpr int BN = SWIGLU ? 64 : 32 * FNW;                         // output columns of a workgroup
   const size_t smem = (size_t)S * (32 * FNW + 128) * T_ROWB;         // also holds the 32 KB that SWIGLU passes between waves
   static bool configured = false;
@@ -798,12 +806,12 @@ static int launch_pipe(elem_t* out, const elem_t* act, const elem_t* w, int M, i
         (void)hipFuncSetAttribute((const void*)gemm_pipe_kernel<S, true, SWIGLU, FNW, 4>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
         touched = true;
       }
-      gemm_pipe_kernel<S, true, SWIGLU, FNW, 4><<<grid, 256, smem, st>>>(out, act, w, M, N, K, lda, ldo, vec_ok, band_w);
+      gemm_pipe_kernel<S, true, SWIGLU, FNW, 4><<<grid, 256, smem, st>>>(out, act, w, M, N, K, lda, ldo, vec_ok, band_w, block_weights, weights_stride);
       return vk_check_launch("gemm_pipe");
     }
   }
-  if (K % KC == 0) gemm_pipe_kernel<S, true, SWIGLU, FNW><<<grid, 256, smem, st>>>(out, act, w, M, N, K, lda, ldo, vec_ok, band_w);
-  else gemm_pipe_kernel<S, false, SWIGLU, FNW><<<grid, 256, smem, st>>>(out, act, w, M, N, K, lda, ldo, vec_ok, band_w);
+  if (K % KC == 0) gemm_pipe_kernel<S, true, SWIGLU, FNW><<<grid, 256, smem, st>>>(out, act, w, M, N, K, lda, ldo, vec_ok, band_w, block_weights, weights_stride);
+  else gemm_pipe_kernel<S, false, SWIGLU, FNW><<<grid, 256, smem, st>>>(out, act, w, M, N, K, lda, ldo, vec_ok, band_w, block_weights, weights_stride);
   return vk_check_launch("gemm_pipe");
 }
 
@@ -1264,6 +1272,21 @@ static int pipe_fragments_by_rounds(int M, int N) {
 }
 
 extern "C" {
+
+// A grouped product through the tile kernel: rows in blocks of 128, block b multiplied by the weight matrix
+// block_weights[b] of several [N, K] matrices that lie weights_stride elements apart (negative: the block is skipped and
+// its output rows are left as they are).  K in whole pairs of slabs (128 bytes of a row).  The same bits as vk_gemm gives
+// for the same rows and matrix.
+int vk_gemm_grouped(elem_t* out, const elem_t* act, const elem_t* w, int M, int N, int K, int64_t lda, int64_t ldo,
+                    const int32_t* block_weights, int64_t weights_stride, hipStream_t st) {
+  VK_REQUIRE(M >= 0 && N > 0 && K > 0 && M % 128 == 0, "grouped gemm: bad sizes M=%d N=%d K=%d (rows in blocks of 128)", M, N, K);
+  VK_REQUIRE(K % (2 * VK_SLAB) == 0, "grouped gemm: K=%d must be a multiple of %d", K, 2 * VK_SLAB);
+  VK_REQUIRE(lda >= K && lda % VK_VEC == 0 && ldo >= N, "grouped gemm: bad row strides");
+  VK_REQUIRE(((uintptr_t)act % 16) == 0 && ((uintptr_t)w % 16) == 0 && block_weights != nullptr && weights_stride % VK_VEC == 0,
+             "grouped gemm: operands must be 16-byte aligned");
+  if (M == 0) return 0;
+  return launch_pipe<2>(out, act, w, M, N, K, lda, ldo, (ldo % 4 == 0) && ((uintptr_t)out % 16 == 0), st, block_weights, weights_stride);
+}
 
 // kernel: 0 = choose by size, 1 = skinny (M <= 64), 2 = tiled (pipelined if K allows), 3 = tiled through
 // registers, 4..6 = pipelined with 2..4 stages, 7 = skinny with two weight tiles per workgroup where it has

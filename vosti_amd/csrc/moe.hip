@@ -1,5 +1,5 @@
 // A mixture of small feed-forward experts, each token through its `top` best of E: the router, the plan that sorts
-// (token, choice) pairs by expert into tiles of 16 rows, the two projections as grouped products on the matrix unit,
+// (token, choice) pairs by expert into tiles of rows, the two projections as grouped products on the matrix unit,
 // and the weighted sum of a token's experts.
 //
 //   z = W_router h (32-bit sums of the elements' exact products);  s = softmax(z) over all experts;  the `top` largest
@@ -102,20 +102,20 @@ __global__ __launch_bounds__(256) void moe_choose_kernel(int32_t* __restrict__ i
   for (int k = 64 + lane; k < top; k += 64) wts[(int64_t)t * top + k] = wts[(int64_t)t * top + k] / denom;
 }
 
-// The plan, by one workgroup.  counts the pairs of every expert, gives expert e the rows [start_e, start_e + 16 *
-// ceil(count_e / 16)) and every pair a row among its expert's (in no fixed order: a row's result does not depend on
+// The plan, by one workgroup.  counts the pairs of every expert, gives expert e the rows [start_e, start_e + tile_rows *
+// ceil(count_e / tile_rows)) and every pair a row among its expert's (in no fixed order: a row's result does not depend on
 // its place).  row_pair [max_rows]: the pair (token * top + choice) of a row, or -1; row_token [max_rows]: the row's
 // token (0 for a row without a pair); pair_row [pairs]; tile_expert [max_tiles]: the expert of a tile, or -1 beyond the
 // last; expert_start [E + 1]: the first row of every expert, and the rows in use.
 __global__ __launch_bounds__(1024) void moe_plan_kernel(const int32_t* __restrict__ idx, int32_t* __restrict__ row_pair,
                                                         int32_t* __restrict__ row_token, int32_t* __restrict__ pair_row,
                                                         int32_t* __restrict__ tile_expert, int32_t* __restrict__ expert_start, int pairs, int top,
-                                                        int E, int max_tiles) {
+                                                        int E, int max_tiles, int tile_rows) {
   extern __shared__ int32_t plan[];      // [E] counts, then [E] cursors
   int32_t* count = plan;
   int32_t* cursor = plan + E;
   for (int e = threadIdx.x; e < E; e += blockDim.x) count[e] = 0;
-  for (int r = threadIdx.x; r < max_tiles * MOE_TILE; r += blockDim.x) {
+  for (int r = threadIdx.x; r < max_tiles * tile_rows; r += blockDim.x) {
     row_pair[r] = -1;
     row_token[r] = 0;
   }
@@ -126,13 +126,13 @@ __global__ __launch_bounds__(1024) void moe_plan_kernel(const int32_t* __restric
   if (threadIdx.x == 0) {
     int tile = 0;
     for (int e = 0; e < E; ++e) {
-      const int n = (count[e] + MOE_TILE - 1) / MOE_TILE;
-      cursor[e] = tile * MOE_TILE;
-      expert_start[e] = tile * MOE_TILE;
+      const int n = (count[e] + tile_rows - 1) / tile_rows;
+      cursor[e] = tile * tile_rows;
+      expert_start[e] = tile * tile_rows;
       for (int j = 0; j < n; ++j) tile_expert[tile + j] = e;
       tile += n;
     }
-    expert_start[E] = tile * MOE_TILE;
+    expert_start[E] = tile * tile_rows;
   }
   __syncthreads();
   for (int i = threadIdx.x; i < pairs; i += blockDim.x) {
@@ -249,11 +249,11 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(float* __restrict__ ou
 
 extern "C" {
 
-// Rows that the plan may need for T tokens: every pair, and up to 15 rows of padding an expert that got any.
-int vk_moe_max_tiles(int T, int top, int E) {
+// Tiles that the plan may need for T tokens: every pair, and up to tile_rows - 1 rows of padding an expert that got any.
+int vk_moe_max_tiles(int T, int top, int E, int tile_rows) {
   const int64_t pairs = (int64_t)T * top;
   const int64_t busy = std::min<int64_t>(E, pairs);
-  return (int)((pairs + busy * (MOE_TILE - 1)) / MOE_TILE);
+  return (int)((pairs + busy * (tile_rows - 1)) / tile_rows);
 }
 
 // logits: scratch [T, E] floats.
@@ -270,11 +270,11 @@ int vk_moe_route(int32_t* idx, float* wts, float* logits, const elem_t* h, const
 }
 
 int vk_moe_plan(const int32_t* idx, int32_t* row_pair, int32_t* row_token, int32_t* pair_row, int32_t* tile_expert, int32_t* expert_start, int T,
-                int top, int E, hipStream_t st) {
-  VK_REQUIRE(T >= 0 && top > 0 && E > 0 && E <= 4096, "expert plan: bad sizes T=%d top=%d E=%d", T, top, E);
+                int top, int E, int tile_rows, hipStream_t st) {
+  VK_REQUIRE(T >= 0 && top > 0 && E > 0 && E <= 4096 && tile_rows > 0, "expert plan: bad sizes T=%d top=%d E=%d", T, top, E);
   if (T == 0) return 0;
   moe_plan_kernel<<<1, 1024, (size_t)2 * E * sizeof(int32_t), st>>>(idx, row_pair, row_token, pair_row, tile_expert, expert_start, T * top, top, E,
-                                                                    vk_moe_max_tiles(T, top, E));
+                                                                    vk_moe_max_tiles(T, top, E, tile_rows), tile_rows);
   return vk_check_launch("expert plan");
 }
 
@@ -285,7 +285,7 @@ int vk_moe_up(elem_t* act, int64_t ldo, const elem_t* x, int64_t ldx, const elem
              "experts (up): bad sizes N=%d K=%d (K in whole 16-byte vectors)", N, K);
   VK_REQUIRE(((uintptr_t)x % 16) == 0 && ((uintptr_t)w_up % 16) == 0, "experts (up): operands must be 16-byte aligned");
   if (T == 0) return 0;
-  const int tiles = vk_moe_max_tiles(T, top, E);
+  const int tiles = vk_moe_max_tiles(T, top, E, MOE_TILE);
   VK_REQUIRE(tiles <= 65535, "experts (up): too many tiles for one launch");
   moe_gemm_kernel<true><<<dim3((N + 15) / 16, tiles), 64 * MOE_WAVES, 0, st>>>(act, ldo, x, ldx, w_up, (int64_t)N * K, row_pair, row_token, tile_expert,
                                                                                N, K);
@@ -299,7 +299,7 @@ int vk_moe_down(elem_t* y, const elem_t* act, int64_t lda, const elem_t* w_down,
              "experts (down): bad sizes N=%d K=%d (K in whole 16-byte vectors)", N, K);
   VK_REQUIRE(((uintptr_t)act % 16) == 0 && ((uintptr_t)w_down % 16) == 0, "experts (down): operands must be 16-byte aligned");
   if (T == 0) return 0;
-  const int tiles = vk_moe_max_tiles(T, top, E);
+  const int tiles = vk_moe_max_tiles(T, top, E, MOE_TILE);
   VK_REQUIRE(tiles <= 65535, "experts (down): too many tiles for one launch");
   moe_gemm_kernel<false><<<dim3((N + 15) / 16, tiles), 64 * MOE_WAVES, 0, st>>>(y, N, act, lda, w_down, (int64_t)N * K, row_pair, nullptr, tile_expert,
                                                                                 N, K);

@@ -7,7 +7,7 @@
 //
 // A sequence's tokens are walked in order by one workgroup per (sequence, head, block of value columns).  A column's
 // state is spread over R neighbouring lanes, each holding DR consecutive state rows in registers; a token's read-out is
-// the sum over a lane's rows in ascending order and then a butterfly over the R lanes, whatever the step's cut: the
+// the sum over a lane's rows in ascending order and then a butterfly over the R lanes (group_sum), whatever the step's cut: the
 // state that a step leaves in memory (per head [P][N], 32-bit) is what the next step starts from, bit for bit.  The
 // inputs of a chunk of tokens go through LDS: the next chunk's are read from global memory into registers before this
 // chunk is walked and written to the other LDS buffer after it (one barrier a chunk).
@@ -69,45 +69,40 @@ __global__ __launch_bounds__(SSM_THREADS) void ssm_scan_kernel(SsmArgs a) {
   const float Dh = load_weight(a.D, a.w_is_f32, h);
 
   float reg[ROUNDS][SSM_CHUNK];
+  float dt_reg = 0.f;
   auto fetch = [&](int c) {
 #pragma unroll
     for (int rd = 0; rd < ROUNDS; ++rd) {
       const int e = tid + rd * SSM_THREADS;
       // Where this thread's element of a token's row comes from: -1 nowhere (padding), else an offset from the row's start.
       int64_t src = -1;
-      bool is_dt = false;
       if (e < NP) { if (e < N) src = a.b_col + g * N + e; }
       else if (e < 2 * NP) { if (e - NP < N) src = a.c_col + g * N + (e - NP); }
       else if (e < 2 * NP + COLS) { if ((int)(blockIdx.z * COLS) + (e - 2 * NP) < P) src = h * P + blockIdx.z * COLS + (e - 2 * NP); }
-      else if (e == L1 - 1) is_dt = true;
 #pragma unroll
       for (int i = 0; i < SSM_CHUNK; ++i) {
         const int t = c * SSM_CHUNK + i;
         float v = 0.f;
-        if (t < n_tok) {
-          const int64_t row = (int64_t)(first + t);
-          if (src >= 0) v = a.xbc[row * a.ldx + src];
-          else if (is_dt) v = to_f32(a.dt[row * a.lddt + h]);
-        }
+        if (t < n_tok && src >= 0) v = a.xbc[(int64_t)(first + t) * a.ldx + src];
         reg[rd][i] = v;
       }
     }
+    // The step sizes: thread i has token i's, so that their softplus and exponentials run side by side.
+    dt_reg = 0.f;
+    if (tid < SSM_CHUNK && c * SSM_CHUNK + tid < n_tok) dt_reg = to_f32(a.dt[(int64_t)(first + c * SSM_CHUNK + tid) * a.lddt + h]);
   };
   auto stage = [&](float* dst) {
 #pragma unroll
     for (int rd = 0; rd < ROUNDS; ++rd) {
       const int e = tid + rd * SSM_THREADS;
-      if (e >= L1) continue;
+      if (e >= L1 - 1) continue;
 #pragma unroll
-      for (int i = 0; i < SSM_CHUNK; ++i) {
-        if (e == L1 - 1) {
-          const float dtv = ssm_softplus(reg[rd][i] + bias);
-          dst[i * RS + e] = dtv;
-          dst[i * RS + e + 1] = expf(-rate * dtv);
-        } else {
-          dst[i * RS + e] = reg[rd][i];
-        }
-      }
+      for (int i = 0; i < SSM_CHUNK; ++i) dst[i * RS + e] = reg[rd][i];
+    }
+    if (tid < SSM_CHUNK) {
+      const float dtv = ssm_softplus(dt_reg + bias);
+      dst[tid * RS + L1 - 1] = dtv;
+      dst[tid * RS + L1] = expf(-rate * dtv);
     }
   };
 
@@ -120,33 +115,44 @@ __global__ __launch_bounds__(SSM_THREADS) void ssm_scan_kernel(SsmArgs a) {
     const float* cur = lds + (c & 1) * (SSM_CHUNK * RS);
     const int m = min(SSM_CHUNK, n_tok - c * SSM_CHUNK);
     float* yout = a.y + (int64_t)(first + c * SSM_CHUNK) * ((int64_t)a.H * P) + (int64_t)h * P + p;
-    for (int i = 0; i < m; ++i) {
-      const float* row = cur + i * RS;
-      const float xv = row[2 * NP + col], dtv = row[L1 - 1], dA = row[L1];
-      const float dx = dtv * xv;
-      const float* Bp = row + r * DR;
-      const float* Cp = row + NP + r * DR;
-      float acc = 0.f;
-      if constexpr (DR % 4 == 0) {
+    // Four tokens at a time: the states move on token by token, the four read-outs' sums over the lanes run side by side.
+    for (int i0 = 0; i0 < m; i0 += 4) {
+      float acc[4], xv[4];
 #pragma unroll
-        for (int q = 0; q < DR / 4; ++q) {
-          const f32x4 b4 = *reinterpret_cast<const f32x4*>(Bp + 4 * q), c4 = *reinterpret_cast<const f32x4*>(Cp + 4 * q);
+      for (int u = 0; u < 4; ++u) {
+        acc[u] = 0.f;
+        xv[u] = 0.f;
+        if (i0 + u < m) {
+          const float* row = cur + (i0 + u) * RS;
+          xv[u] = row[2 * NP + col];
+          const float dtv = row[L1 - 1], dA = row[L1];
+          const float dx = dtv * xv[u];
+          const float* Bp = row + r * DR;
+          const float* Cp = row + NP + r * DR;
+          if constexpr (DR % 4 == 0) {
 #pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            S[4 * q + j] = __builtin_fmaf(dA, S[4 * q + j], dx * b4[j]);
-            acc = __builtin_fmaf(S[4 * q + j], c4[j], acc);
+            for (int q = 0; q < DR / 4; ++q) {
+              const f32x4 b4 = *reinterpret_cast<const f32x4*>(Bp + 4 * q), c4 = *reinterpret_cast<const f32x4*>(Cp + 4 * q);
+#pragma unroll
+              for (int j = 0; j < 4; ++j) {
+                S[4 * q + j] = __builtin_fmaf(dA, S[4 * q + j], dx * b4[j]);
+                acc[u] = __builtin_fmaf(S[4 * q + j], c4[j], acc[u]);
+              }
+            }
+          } else {
+#pragma unroll
+            for (int j = 0; j < DR; ++j) {
+              S[j] = __builtin_fmaf(dA, S[j], dx * Bp[j]);
+              acc[u] = __builtin_fmaf(S[j], Cp[j], acc[u]);
+            }
           }
-        }
-      } else {
-#pragma unroll
-        for (int j = 0; j < DR; ++j) {
-          S[j] = __builtin_fmaf(dA, S[j], dx * Bp[j]);
-          acc = __builtin_fmaf(S[j], Cp[j], acc);
         }
       }
 #pragma unroll
-      for (int off = 1; off < R; off <<= 1) acc = acc + __shfl_xor(acc, off, VK_WAVE);
-      if (r == 0 && col_ok) yout[(int64_t)i * ((int64_t)a.H * P)] = acc + Dh * xv;
+      for (int u = 0; u < 4; ++u) acc[u] = group_sum<R>(acc[u]);
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+        if (r == 0 && col_ok && i0 + u < m) yout[(int64_t)(i0 + u) * ((int64_t)a.H * P)] = acc[u] + Dh * xv[u];
     }
     if (c + 1 < chunks) stage(lds + ((c + 1) & 1) * (SSM_CHUNK * RS));
     __syncthreads();
@@ -215,7 +221,7 @@ int vk_ssm_scan(float* y, const float* xbc, int64_t ldx, int b_col, int c_col, c
   do {                                                                                                                           \
     constexpr int cols = SSM_THREADS / (R);                                                                                      \
     const size_t smem = (size_t)2 * SSM_CHUNK * (2 * (R) * (DR) + cols + 4) * sizeof(float);                                      \
-    static_assert((2 * (R) * (DR) + cols + 1 + SSM_THREADS - 1) / SSM_THREADS <= (ROUNDS), "a round more is needed");            \
+    static_assert((2 * (R) * (DR) + cols + SSM_THREADS - 1) / SSM_THREADS <= (ROUNDS), "a round more is needed");            \
     static bool raised = false;                                                                                                  \
     if (!raised && smem > 48 * 1024) {                                                                                           \
       (void)hipFuncSetAttribute((const void*)ssm_scan_kernel<R, DR, ROUNDS>, hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024); \
