@@ -120,7 +120,7 @@ struct Kernels::Fn {
   int (*embed_scaled)(P, CP, CP, int, int, int, float, hipStream_t);
   int (*stream_add)(P, CP, CP, int, CP, int, int64_t, hipStream_t);
   int (*stream_pair_norm)(P, CP, CP, CP, CP, int, int, int, float, float, float, hipStream_t);
-  int (*ssm_scan)(P, CP, int64_t, int, int, CP, int64_t, CP, CP, CP, int, P, int64_t, CP, CP, CP, int, int, int, int, int, hipStream_t);
+  int (*ssm_scan)(P, CP, int64_t, int, int, CP, int64_t, CP, CP, CP, int, P, int64_t, CP, CP, CP, int, int, int, int, int, int, hipStream_t);
   int (*ssm_gate_norm)(P, int64_t, CP, CP, int64_t, CP, int, int, int, int, float, hipStream_t);
   int (*moe_max_tiles)(int, int, int, int);
   int (*gemm_grouped)(P, CP, CP, int, int, int, int64_t, int64_t, CP, int64_t, hipStream_t);
@@ -719,8 +719,8 @@ Tensor Kernels::ssm_scan(const Tensor& xbc, int64_t b_col, int64_t c_col, const 
   expect(slots, "state slots", DType::I32, {S});
   Tensor y = empty({T, H, P}, DType::F32);
   call(fn_->ssm_scan(y.data, xbc.data, xbc.dim(1), (int)b_col, (int)c_col, static_cast<const char*>(proj.data) + (size_t)dt_col * dtype_bytes(dtype_),
-                     proj.dim(1), dt_bias.data, A_log.data, D.data, wf, state.data, state.dim(1), cu_q.data, positions.data, slots.data, (int)S, H, G,
-                     N, P, stream));
+                     proj.dim(1), dt_bias.data, A_log.data, D.data, wf, state.data, state.dim(1), cu_q.data, positions.data, slots.data, (int)S, (int)T, H,
+                     G, N, P, stream));
   return y;
 }
 

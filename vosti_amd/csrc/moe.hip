@@ -31,6 +31,7 @@ __global__ __launch_bounds__(256) void moe_logits_kernel(float* __restrict__ z, 
 #pragma unroll
   for (int i = 0; i < MOE_ROUTE_TOKENS; ++i) acc[i] = 0.f;
   const elem_t* wr = router + (int64_t)e * W;
+#pragma unroll 4
   for (int c = lane * VK_VEC; c < W; c += 64 * VK_VEC) {
     float wv[VK_VEC];
     load_elems(wr + c, wv);
@@ -228,12 +229,19 @@ __global__ __launch_bounds__(64 * MOE_WAVES) void moe_gemm_kernel(elem_t* __rest
   }
 }
 
-// x <- max(x, 0)^2, element by element: the experts' activation on a product that was left as elements.
-__global__ __launch_bounds__(256) void moe_relu_square_kernel(elem_t* x, int64_t n) {
+// x <- max(x, 0)^2, element by element: the experts' activation on a product that was left as elements.  A thread
+// takes a 16-byte vector (n in whole vectors).
+__global__ __launch_bounds__(256) void moe_relu_square_kernel(elem_t* x, int64_t nvec) {
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= n) return;
-  const float rl = fmaxf(to_f32(x[i]), 0.f);
-  x[i] = from_f32<elem_t>(rl * rl);
+  if (i >= nvec) return;
+  float v[VK_VEC];
+  load_elems(x + i * VK_VEC, v);
+#pragma unroll
+  for (int j = 0; j < VK_VEC; ++j) {
+    const float rl = fmaxf(v[j], 0.f);
+    v[j] = rl * rl;
+  }
+  store_elems(x + i * VK_VEC, v);
 }
 
 // out[t, c] = sum over k < top, ascending, of wts[t, k] * y[pair_row[t * top + k], c], from zero.
@@ -307,9 +315,10 @@ int vk_moe_down(elem_t* y, const elem_t* act, int64_t lda, const elem_t* w_down,
 }
 
 int vk_moe_relu_square(elem_t* x, int64_t n, hipStream_t st) {
-  VK_REQUIRE(n >= 0, "experts (activation): bad size");
+  VK_REQUIRE(n >= 0 && n % VK_VEC == 0 && ((uintptr_t)x % 16) == 0, "experts (activation): whole 16-byte vectors are needed");
   if (n == 0) return 0;
-  moe_relu_square_kernel<<<(unsigned)((n + 255) / 256), 256, 0, st>>>(x, n);
+  const int64_t nvec = n / VK_VEC;
+  moe_relu_square_kernel<<<(unsigned)((nvec + 255) / 256), 256, 0, st>>>(x, nvec);
   return vk_check_launch("experts (activation)");
 }
 

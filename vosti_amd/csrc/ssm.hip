@@ -41,8 +41,10 @@ struct SsmArgs {
 __device__ __forceinline__ float ssm_softplus(float z) { return z > 20.f ? z : log1pf(expf(z)); }
 
 // R lanes share a value column, each with DR consecutive state rows; a workgroup has 256 / R columns.  In LDS the
-// state rows are padded with zeros to R * DR, so that no lane has to ask whether a row exists.
-template <int R, int DR, int ROUNDS>
+// state rows are padded with zeros to R * DR, so that no lane has to ask whether a row exists.  CH: tokens a chunk (16,
+// or 1 for a step of single tokens, whose workgroups then need little LDS and all run at once; the arithmetic of a token
+// is the same).
+template <int R, int DR, int ROUNDS, int CH>
 __global__ __launch_bounds__(SSM_THREADS) void ssm_scan_kernel(SsmArgs a) {
   extern __shared__ float lds[];
   constexpr int COLS = SSM_THREADS / R, NP = R * DR;
@@ -68,7 +70,7 @@ __global__ __launch_bounds__(SSM_THREADS) void ssm_scan_kernel(SsmArgs a) {
   const float rate = expf(load_weight(a.A_log, a.w_is_f32, h));
   const float Dh = load_weight(a.D, a.w_is_f32, h);
 
-  float reg[ROUNDS][SSM_CHUNK];
+  float reg[ROUNDS][CH];
   float dt_reg = 0.f;
   auto fetch = [&](int c) {
 #pragma unroll
@@ -80,8 +82,8 @@ __global__ __launch_bounds__(SSM_THREADS) void ssm_scan_kernel(SsmArgs a) {
       else if (e < 2 * NP) { if (e - NP < N) src = a.c_col + g * N + (e - NP); }
       else if (e < 2 * NP + COLS) { if ((int)(blockIdx.z * COLS) + (e - 2 * NP) < P) src = h * P + blockIdx.z * COLS + (e - 2 * NP); }
 #pragma unroll
-      for (int i = 0; i < SSM_CHUNK; ++i) {
-        const int t = c * SSM_CHUNK + i;
+      for (int i = 0; i < CH; ++i) {
+        const int t = c * CH + i;
         float v = 0.f;
         if (t < n_tok && src >= 0) v = a.xbc[(int64_t)(first + t) * a.ldx + src];
         reg[rd][i] = v;
@@ -89,7 +91,7 @@ __global__ __launch_bounds__(SSM_THREADS) void ssm_scan_kernel(SsmArgs a) {
     }
     // The step sizes: thread i has token i's, so that their softplus and exponentials run side by side.
     dt_reg = 0.f;
-    if (tid < SSM_CHUNK && c * SSM_CHUNK + tid < n_tok) dt_reg = to_f32(a.dt[(int64_t)(first + c * SSM_CHUNK + tid) * a.lddt + h]);
+    if (tid < CH && c * CH + tid < n_tok) dt_reg = to_f32(a.dt[(int64_t)(first + c * CH + tid) * a.lddt + h]);
   };
   auto stage = [&](float* dst) {
 #pragma unroll
@@ -97,24 +99,24 @@ __global__ __launch_bounds__(SSM_THREADS) void ssm_scan_kernel(SsmArgs a) {
       const int e = tid + rd * SSM_THREADS;
       if (e >= L1 - 1) continue;
 #pragma unroll
-      for (int i = 0; i < SSM_CHUNK; ++i) dst[i * RS + e] = reg[rd][i];
+      for (int i = 0; i < CH; ++i) dst[i * RS + e] = reg[rd][i];
     }
-    if (tid < SSM_CHUNK) {
+    if (tid < CH) {
       const float dtv = ssm_softplus(dt_reg + bias);
       dst[tid * RS + L1 - 1] = dtv;
       dst[tid * RS + L1] = expf(-rate * dtv);
     }
   };
 
-  const int chunks = (n_tok + SSM_CHUNK - 1) / SSM_CHUNK;
+  const int chunks = (n_tok + CH - 1) / CH;
   fetch(0);
   stage(lds);
   __syncthreads();
   for (int c = 0; c < chunks; ++c) {
     if (c + 1 < chunks) fetch(c + 1);
-    const float* cur = lds + (c & 1) * (SSM_CHUNK * RS);
-    const int m = min(SSM_CHUNK, n_tok - c * SSM_CHUNK);
-    float* yout = a.y + (int64_t)(first + c * SSM_CHUNK) * ((int64_t)a.H * P) + (int64_t)h * P + p;
+    const float* cur = lds + (c & 1) * (CH * RS);
+    const int m = min(CH, n_tok - c * CH);
+    float* yout = a.y + (int64_t)(first + c * CH) * ((int64_t)a.H * P) + (int64_t)h * P + p;
     // Four tokens at a time: the states move on token by token, the four read-outs' sums over the lanes run side by side.
     for (int i0 = 0; i0 < m; i0 += 4) {
       float acc[4], xv[4];
@@ -154,7 +156,7 @@ __global__ __launch_bounds__(SSM_THREADS) void ssm_scan_kernel(SsmArgs a) {
       for (int u = 0; u < 4; ++u)
         if (r == 0 && col_ok && i0 + u < m) yout[(int64_t)(i0 + u) * ((int64_t)a.H * P)] = acc[u] + Dh * xv[u];
     }
-    if (c + 1 < chunks) stage(lds + ((c + 1) & 1) * (SSM_CHUNK * RS));
+    if (c + 1 < chunks) stage(lds + ((c + 1) & 1) * (CH * RS));
     __syncthreads();
   }
   if (col_ok) {
@@ -201,10 +203,11 @@ extern "C" {
 
 // y [T, H, P] floats.  xbc: float rows of length ldx with x (H heads of P) from column 0, B (G groups of N) from b_col
 // and C from c_col; dt: elements, the step size's pre-activation of head h at dt[t * lddt + h]; dt_bias, A_log, D: [H]
-// (all floats or all elements).  state: per slot, the H states at its start, each [P][N].
+// (all floats or all elements).  state: per slot, the H states at its start, each [P][N].  T: the rows of y (every one of
+// the S sequences brings at least one).
 int vk_ssm_scan(float* y, const float* xbc, int64_t ldx, int b_col, int c_col, const elem_t* dt, int64_t lddt, const void* dt_bias,
                 const void* A_log, const void* D, int w_is_f32, float* state, int64_t state_stride, const int32_t* cu_q,
-                const int32_t* positions, const int32_t* slots, int S, int H, int G, int N, int P, hipStream_t st) {
+                const int32_t* positions, const int32_t* slots, int S, int T, int H, int G, int N, int P, hipStream_t st) {
   VK_REQUIRE(S >= 0 && H > 0 && G > 0 && H % G == 0 && N > 0 && N <= 256 && P > 0, "state-space scan: bad sizes H=%d G=%d N=%d P=%d (N at most 256)",
              H, G, N, P);
   VK_REQUIRE(b_col >= H * P && c_col >= 0 && ldx >= (int64_t)std::max(b_col, c_col) + (int64_t)G * N && lddt >= H,
@@ -212,6 +215,7 @@ int vk_ssm_scan(float* y, const float* xbc, int64_t ldx, int b_col, int c_col, c
   VK_REQUIRE(state_stride >= (int64_t)H * P * N, "state-space scan: the state does not hold the heads");
   VK_REQUIRE(H <= 65535, "state-space scan: too many heads");
   if (S == 0) return 0;
+  const bool single_tokens = T == S;       // every sequence brings one token
   SsmArgs a;
   a.y = y; a.xbc = xbc; a.ldx = ldx; a.b_col = b_col; a.c_col = c_col; a.dt = dt; a.lddt = lddt; a.dt_bias = dt_bias; a.A_log = A_log; a.D = D;
   a.w_is_f32 = w_is_f32; a.state = state; a.state_stride = state_stride; a.cu_q = cu_q; a.positions = positions; a.slots = slots;
@@ -220,15 +224,20 @@ int vk_ssm_scan(float* y, const float* xbc, int64_t ldx, int b_col, int c_col, c
 #define SSM_SCAN(R, DR, ROUNDS)                                                                                                  \
   do {                                                                                                                           \
     constexpr int cols = SSM_THREADS / (R);                                                                                      \
-    const size_t smem = (size_t)2 * SSM_CHUNK * (2 * (R) * (DR) + cols + 4) * sizeof(float);                                      \
-    static_assert((2 * (R) * (DR) + cols + SSM_THREADS - 1) / SSM_THREADS <= (ROUNDS), "a round more is needed");            \
-    static bool raised = false;                                                                                                  \
-    if (!raised && smem > 48 * 1024) {                                                                                           \
-      (void)hipFuncSetAttribute((const void*)ssm_scan_kernel<R, DR, ROUNDS>, hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024); \
-      raised = true;                                                                                                             \
-    }                                                                                                                            \
+    static_assert((2 * (R) * (DR) + cols + SSM_THREADS - 1) / SSM_THREADS <= (ROUNDS), "a round more is needed");                \
     VK_REQUIRE((P + cols - 1) / cols <= 65535, "state-space scan: too many columns");                                            \
-    ssm_scan_kernel<R, DR, ROUNDS><<<dim3(S, H, (P + cols - 1) / cols), SSM_THREADS, smem, st>>>(a);                             \
+    const dim3 grid(S, H, (P + cols - 1) / cols);                                                                                \
+    if (single_tokens) {                                                                                                         \
+      ssm_scan_kernel<R, DR, ROUNDS, 1><<<grid, SSM_THREADS, (size_t)2 * (2 * (R) * (DR) + cols + 4) * sizeof(float), st>>>(a);   \
+    } else {                                                                                                                     \
+      const size_t smem = (size_t)2 * SSM_CHUNK * (2 * (R) * (DR) + cols + 4) * sizeof(float);                                    \
+      static bool raised = false;                                                                                                \
+      if (!raised && smem > 48 * 1024) {                                                                                         \
+        (void)hipFuncSetAttribute((const void*)ssm_scan_kernel<R, DR, ROUNDS, SSM_CHUNK>, hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024); \
+        raised = true;                                                                                                           \
+      }                                                                                                                          \
+      ssm_scan_kernel<R, DR, ROUNDS, SSM_CHUNK><<<grid, SSM_THREADS, smem, st>>>(a);                                             \
+    }                                                                                                                            \
   } while (0)
   if (N <= 8) SSM_SCAN(8, 1, 1);
   else if (N <= 16) SSM_SCAN(8, 2, 1);
