@@ -534,13 +534,13 @@ def tezinex_config(width, heads, kv_heads, ff, layers, vocab):
 
 def povatar_config(width, heads, kv_heads, ff, layers, vocab):
     """Every layer: attention (heads of 128, keys of the query's own block of 1,024 positions, half of every head rotated
-    with stretched frequencies) beside a state-space recurrence as wide as the model (heads of 64, 128 state rows), and 16
-    experts of which a token uses 2, each half as wide as the dense feed-forward of the same size: a token's matrix work
-    is that of a Tezinex or Qwen3 layer of these sizes, plus the recurrence's projections."""
+    with stretched frequencies) beside a state-space recurrence as wide as the model (heads of 64, 128 state rows), and 32
+    experts of which a token uses 4, each a quarter as wide as the dense feed-forward of the same size: a token's matrix
+    work is that of a Tezinex or Qwen3 layer of these sizes, plus the recurrence's projections."""
     left = {"dim": 128, "vdim": 128, "heads": heads, "kv_heads": kv_heads, "mask": {"size": 1024}, "scale": 128 ** -0.5,
-            "rot": {"base": 10000.0, "dims": 64, "scaling": {"factor": 8.0, "fast": 32.0, "original": 4096, "slow": 1.0}}}
-    right = {"conv": 4, "groups": 2, "heads": width // 64, "norm_groups": 2, "state": 128, "vdim": 64}
-    mlp = {"kind": "moe", "expert": {"ff": ff // 2}, "router": {"experts": 16, "top": 2}}
+            "rot": {"base": 10000.0, "dims": 64, "scaling": {"factor": 4.0, "fast": 16.0, "original": 4096, "slow": 2.0}}}
+    right = {"conv": 4, "groups": 4, "heads": width // 64, "norm_groups": 4, "state": 128, "vdim": 64}
+    mlp = {"kind": "moe", "expert": {"ff": ff // 4}, "router": {"experts": 32, "top": 4}}
     return {"architecture": "Povatar", "embedding": {"scale": 1.0}, "norm": {"eps": 1e-5}, "vocab": vocab, "width": width,
             "layers": [{"type": "parallel", "mixer": {"left": left, "right": right}, "mlp": mlp} for _ in range(layers)]}
 
@@ -560,7 +560,7 @@ def tezinex_workload(args) -> dict:
     record = {"metric": "decode_tokens_per_s", "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
               "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if args.dtype == "bfloat16" else "fp32",
               "data": "synthetic: seeded random token prompts, seeded random weights", "sizes": {},
-              "config": {"model": "Povatar (attention beside a state-space recurrence, 16 experts of which 2) beside Tezinex at equal size"
+              "config": {"model": "Povatar (attention beside a state-space recurrence, 32 experts of which 4) beside Tezinex at equal size"
                          if args.workload == "povatar" else "Tezinex (delta, attention, shared-key attention, delta, ...) beside Qwen3 at equal size",
                          "layers": layers,
                          "global_batch": batch, "seq_len": prompt_tokens, "vocab_size": vocab, "parallelism": "single GPU",

@@ -45,7 +45,7 @@ MIXED = config([
     layer(left(2, 1, 48, 16, size=64, rot_dims=16), right(6, 4, 8, 3, 3, conv=1), moe(1, 1, 16)),
 ], width=64, vocab=97)
 # One layer with the head size of the kernels' widest tiles and a state as wide as a wave.
-WIDE = config([layer(left(4, 2, 128, 128, size=150, rot_dims=64, scaling={"factor": 8.0, "fast": 32.0, "original": 256, "slow": 1.0}),
+WIDE = config([layer(left(4, 2, 128, 128, size=150, rot_dims=64, scaling={"factor": 6.0, "fast": 20.0, "original": 256, "slow": 1.5}),
                      right(2, 64, 64, 1, 2, conv=4), moe(8, 2, 72))], width=96, vocab=130, embed_scale=9.0)
 CONFIGS = {"MIXED": MIXED, "WIDE": WIDE}
 

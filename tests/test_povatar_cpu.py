@@ -82,7 +82,7 @@ def test_tensor_names_are_the_files(tmp_path):
 
 @pytest.mark.parametrize("rot", [
     {"base": 10000.0, "dims": 8, "scaling": STRETCH},
-    {"base": 20000.0, "dims": 64, "scaling": {"factor": 8.0, "fast": 32.0, "original": 4096, "slow": 1.0}},
+    {"base": 50000.0, "dims": 64, "scaling": {"factor": 6.0, "fast": 24.0, "original": 4096, "slow": 1.5}},
     {"base": 300.0, "dims": 6, "scaling": {"factor": 2.0, "fast": 4.0, "original": 16, "slow": 1.0}},
     {"base": 500.0, "dims": 32},
 ])
