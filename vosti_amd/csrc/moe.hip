@@ -19,20 +19,21 @@
 #define MOE_TILE 16          // rows of a tile: pairs of one expert
 #define MOE_ROUTE_TOKENS 8   // tokens a router workgroup shares an expert's weights among
 
-// Router logits z [T, E] floats.  A workgroup of four waves takes MOE_ROUTE_TOKENS tokens and four experts, a wave one
-// expert for all of them: lane l owns the 16-byte vectors l, l + 64, ... of a row, its products are added in ascending
-// order (fused multiply-adds), then a butterfly over the lanes: the order depends on the width alone.
+// Router logits z [T, E] floats.  A workgroup of four waves takes MOE_ROUTE_TOKENS tokens and one expert; the waves
+// split the row's 16-byte vectors (vector v goes to wave (v / 64) % 4, lane v % 64), a lane adds its products in ascending
+// order (fused multiply-adds), a butterfly follows over the lanes and the four waves' sums are added in wave order: the
+// order depends on the width alone.
 __global__ __launch_bounds__(256) void moe_logits_kernel(float* __restrict__ z, const elem_t* __restrict__ h, const elem_t* __restrict__ router,
                                                          int T, int W, int E) {
+  __shared__ float part[4][MOE_ROUTE_TOKENS];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-  const int t0 = blockIdx.x * MOE_ROUTE_TOKENS, e = blockIdx.y * 4 + wave;
-  if (e >= E) return;
+  const int t0 = blockIdx.x * MOE_ROUTE_TOKENS, e = blockIdx.y;
   float acc[MOE_ROUTE_TOKENS];
 #pragma unroll
   for (int i = 0; i < MOE_ROUTE_TOKENS; ++i) acc[i] = 0.f;
   const elem_t* wr = router + (int64_t)e * W;
-#pragma unroll 4
-  for (int c = lane * VK_VEC; c < W; c += 64 * VK_VEC) {
+#pragma unroll 2
+  for (int c = threadIdx.x * VK_VEC; c < W; c += 256 * VK_VEC) {
     float wv[VK_VEC];
     load_elems(wr + c, wv);
 #pragma unroll
@@ -46,7 +47,15 @@ __global__ __launch_bounds__(256) void moe_logits_kernel(float* __restrict__ z, 
 #pragma unroll
   for (int i = 0; i < MOE_ROUTE_TOKENS; ++i) {
     const float v = wave_sum_xor(acc[i]);
-    if (lane == 0 && t0 + i < T) z[(int64_t)(t0 + i) * E + e] = v;
+    if (lane == 0) part[wave][i] = v;
+  }
+  __syncthreads();
+  if (threadIdx.x < MOE_ROUTE_TOKENS && t0 + (int)threadIdx.x < T) {
+    float v = part[0][threadIdx.x];
+    v = v + part[1][threadIdx.x];
+    v = v + part[2][threadIdx.x];
+    v = v + part[3][threadIdx.x];
+    z[(int64_t)(t0 + threadIdx.x) * E + e] = v;
   }
 }
 
@@ -271,7 +280,7 @@ int vk_moe_route(int32_t* idx, float* wts, float* logits, const elem_t* h, const
              "router: bad sizes T=%d W=%d E=%d top=%d (the width in whole 16-byte vectors, at most 4096 experts)", T, W, E, top);
   VK_REQUIRE(((uintptr_t)h % 16) == 0 && ((uintptr_t)router % 16) == 0, "router: operands must be 16-byte aligned");
   if (T == 0) return 0;
-  moe_logits_kernel<<<dim3((T + MOE_ROUTE_TOKENS - 1) / MOE_ROUTE_TOKENS, (E + 3) / 4), 256, 0, st>>>(logits, h, router, T, W, E);
+  moe_logits_kernel<<<dim3((T + MOE_ROUTE_TOKENS - 1) / MOE_ROUTE_TOKENS, E), 256, 0, st>>>(logits, h, router, T, W, E);
   if (vk_check_launch("router (logits)")) return 1;
   moe_choose_kernel<<<(T + 3) / 4, 256, (size_t)4 * E * sizeof(float), st>>>(idx, wts, logits, T, E, top, weight_eps);
   return vk_check_launch("router (choice)");
